@@ -1,0 +1,232 @@
+"""ctypes/numpy front end of the CPU oracle (``liboracle.so``).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by ``__graft_entry__.smoke()`` and
+by ``bench.py``'s cpu_baseline leg.  Nothing under ``sphconv_amd/`` imports it.
+
+Every function takes and returns numpy arrays in the reference's layouts
+(feature [N,C] float32, z_idx [N] int32, z_ptr [B,S0,S1] int32 inclusive scan,
+rules [NTile,KV,2,tile_n_max] int32 padded with -1, rule_size [NTile,KV]).
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+
+class Geom(C.Structure):
+    _fields_ = [(n, C.c_int) for n in
+                ("B", "S0", "S1", "S2", "O0", "O1", "O2", "K0", "K1", "K2",
+                 "s0", "s1", "s2", "p0", "p1", "p2", "d0", "d1", "d2", "T0", "T1")]
+
+
+def build(force: bool = False) -> str:
+    so = os.path.join(_HERE, "liboracle.so")
+    src = os.path.join(_HERE, "sphconv_oracle.c")
+    if force or not os.path.exists(so) or os.path.getmtime(so) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"],
+                              stdout=subprocess.DEVNULL)
+    return so
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        so = os.path.join(_HERE, "liboracle.so")
+        if not os.path.exists(so):
+            build()
+        _LIB = C.CDLL(so)
+        _LIB.orc_tile_n_max.restype = C.c_int
+        _LIB.orc_in_tile_size.restype = C.c_int
+        _LIB.orc_out_spatial_dim.restype = C.c_int
+        _LIB.orc_num_threads.restype = C.c_int
+    return _LIB
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _i32(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def num_threads() -> int:
+    return lib().orc_num_threads()
+
+
+def set_num_threads(n: int):
+    lib().orc_set_num_threads(int(n))
+
+
+def out_spatial(in_shape, kernel, stride, padding, dilation=(1, 1, 1)):
+    L = lib()
+    return [L.orc_out_spatial_dim(int(i), int(k), int(s), int(p), int(d))
+            for i, k, s, p, d in zip(in_shape, kernel, stride, padding, dilation)]
+
+
+def tile_n_max(B, in_shape, kernel, stride, tile, nnz) -> int:
+    L = lib()
+    it0 = L.orc_in_tile_size(int(tile[0]), int(stride[0]), int(kernel[0]))
+    it1 = L.orc_in_tile_size(int(tile[1]), int(stride[1]), int(kernel[1]))
+    return L.orc_tile_n_max(it0, it1, int(B), int(in_shape[0]), int(in_shape[1]),
+                            int(in_shape[2]), int(nnz))
+
+
+def make_geom(B, in_shape, out_shape, kernel, stride, padding, dilation=(1, 1, 1), tile=(2, 2)):
+    return Geom(int(B), *map(int, in_shape), *map(int, out_shape), *map(int, kernel),
+                *map(int, stride), *map(int, padding), *map(int, dilation), *map(int, tile))
+
+
+def init_tensor(feature, indices, B, shape):
+    """-> (out_feature, z_idx, z_ptr, permutation); fibers sorted by S2."""
+    feature = _f32(feature)
+    indices = _i32(indices)
+    n, c = feature.shape
+    S0, S1, S2 = map(int, shape)
+    out = np.empty_like(feature)
+    z_idx = np.empty(n, np.int32)
+    z_ptr = np.empty((B, S0, S1), np.int32)
+    perm = np.empty(n, np.int32)
+    rc = lib().orc_init_tensor(_p(feature), _p(indices), n, c, int(B), S0, S1, S2,
+                               _p(out), _p(z_idx), _p(z_ptr), _p(perm))
+    if rc:
+        raise ValueError({-1: "coordinate out of range", -2: "duplicate coordinate",
+                          -3: "out of memory"}[rc])
+    return out, z_idx, z_ptr, perm
+
+
+def init_tensor_backward(d_out, perm):
+    d_out = _f32(d_out)
+    perm = _i32(perm)
+    res = np.empty_like(d_out)
+    lib().orc_init_tensor_backward(_p(d_out), _p(perm), d_out.shape[0], d_out.shape[1], _p(res))
+    return res
+
+
+def to_dense(feature, z_idx, z_ptr, S2):
+    """-> [B,S0,S1,S2,C] float32, zeros where inactive."""
+    feature, z_idx, z_ptr = _f32(feature), _i32(z_idx), _i32(z_ptr)
+    B, S0, S1 = z_ptr.shape
+    out = np.zeros((B, S0, S1, int(S2), feature.shape[1]), np.float32)
+    lib().orc_to_dense(_p(feature), _p(z_idx), _p(z_ptr), B, S0, S1, int(S2),
+                       feature.shape[1], _p(out))
+    return out
+
+
+def to_dense_backward(d_out, z_idx, z_ptr):
+    d_out, z_idx, z_ptr = _f32(d_out), _i32(z_idx), _i32(z_ptr)
+    B, S0, S1, S2, c = d_out.shape
+    res = np.zeros((z_idx.shape[0], c), np.float32)
+    lib().orc_to_dense_backward(_p(d_out), _p(z_idx), _p(z_ptr), B, S0, S1, S2, c, _p(res))
+    return res
+
+
+def get_rules_subm(z_idx, z_ptr, B, in_shape, out_shape, kernel, stride, padding,
+                   dilation=(1, 1, 1), tile=(2, 2), n_max=None, canonical=True):
+    """-> (z_idx, z_ptr, rules, rule_size, dropped)."""
+    z_idx, z_ptr = _i32(z_idx), _i32(z_ptr)
+    g = make_geom(B, in_shape, out_shape, kernel, stride, padding, dilation, tile)
+    kv = int(np.prod(kernel))
+    ntile = -(-out_shape[0] // tile[0]) * -(-out_shape[1] // tile[1])
+    if n_max is None:
+        n_max = tile_n_max(B, in_shape, kernel, stride, tile, z_idx.shape[0])
+    grid = np.empty(int(B) * int(np.prod(out_shape)), np.int32)
+    rules = np.empty((ntile, kv, 2, n_max), np.int32)
+    rule_size = np.empty((ntile, kv), np.int32)
+    lib().orc_rules_subm.restype = C.c_int
+    dropped = lib().orc_rules_subm(_p(z_idx), _p(z_ptr), C.byref(g), int(n_max),
+                                   _p(grid), _p(rules), _p(rule_size))
+    if canonical:
+        lib().orc_rules_canonicalize(_p(rules), _p(rule_size), ntile, kv, int(n_max))
+    return z_idx, z_ptr, rules, rule_size, dropped
+
+
+def get_rules(z_idx, z_ptr, B, in_shape, out_shape, kernel, stride, padding,
+              dilation=(1, 1, 1), tile=(2, 2), n_max=None, canonical=True):
+    """-> (oz_idx, oz_ptr, rules, rule_size, dropped)."""
+    z_idx, z_ptr = _i32(z_idx), _i32(z_ptr)
+    g = make_geom(B, in_shape, out_shape, kernel, stride, padding, dilation, tile)
+    kv = int(np.prod(kernel))
+    ntile = -(-out_shape[0] // tile[0]) * -(-out_shape[1] // tile[1])
+    if n_max is None:
+        n_max = tile_n_max(B, in_shape, kernel, stride, tile, z_idx.shape[0])
+    grid = np.empty(int(B) * int(np.prod(out_shape)), np.int32)
+    oz_ptr = np.empty((int(B), int(out_shape[0]), int(out_shape[1])), np.int32)
+    L = lib()
+    L.orc_rules_std_outgrid.restype = C.c_int
+    L.orc_rules_std_fill.restype = C.c_int
+    out_nnz = L.orc_rules_std_outgrid(_p(z_idx), _p(z_ptr), C.byref(g), _p(grid), _p(oz_ptr))
+    oz_idx = np.empty(out_nnz, np.int32)
+    rules = np.empty((ntile, kv, 2, n_max), np.int32)
+    rule_size = np.empty((ntile, kv), np.int32)
+    dropped = L.orc_rules_std_fill(_p(z_idx), _p(z_ptr), C.byref(g), int(n_max), _p(grid),
+                                   _p(oz_idx), _p(rules), _p(rule_size))
+    if canonical:
+        L.orc_rules_canonicalize(_p(rules), _p(rule_size), ntile, kv, int(n_max))
+    return oz_idx, oz_ptr, rules, rule_size, dropped
+
+
+def rule_conv(feature, weight, rules, rule_size, out_nnz):
+    """fp32 forward; weight [KV,iC,oC]."""
+    feature, weight = _f32(feature), _f32(weight)
+    rules, rule_size = _i32(rules), _i32(rule_size)
+    ntile, kv, _, n_max = rules.shape
+    ic, oc = weight.shape[1], weight.shape[2]
+    out = np.empty((int(out_nnz), oc), np.float32)
+    lib().orc_rule_conv_f32(_p(feature), _p(weight), _p(rules), _p(rule_size), ntile, kv,
+                            n_max, ic, oc, int(out_nnz), _p(out))
+    return out
+
+
+def rule_conv_d_feature(d_out, weight_oc_ic, rules, rule_size, tile_grid_shape, nnz):
+    """fp32 dgrad; weight already permuted to [KV,oC,iC] as the reference's caller does."""
+    d_out, w = _f32(d_out), _f32(weight_oc_ic)
+    rules, rule_size = _i32(rules), _i32(rule_size)
+    _, kv, _, n_max = rules.shape
+    oc, ic = w.shape[1], w.shape[2]
+    res = np.empty((int(nnz), ic), np.float32)
+    lib().orc_rule_conv_dfeature_f32(_p(d_out), _p(w), _p(rules), _p(rule_size),
+                                     int(tile_grid_shape[0]), int(tile_grid_shape[1]), kv,
+                                     n_max, ic, oc, int(nnz), _p(res))
+    return res
+
+
+def rule_conv_d_weight(feature, d_out, rules, rule_size):
+    feature, d_out = _f32(feature), _f32(d_out)
+    rules, rule_size = _i32(rules), _i32(rule_size)
+    ntile, kv, _, n_max = rules.shape
+    ic, oc = feature.shape[1], d_out.shape[1]
+    res = np.empty((kv, ic, oc), np.float32)
+    lib().orc_rule_conv_dweight_f32(_p(feature), _p(d_out), _p(rules), _p(rule_size), ntile,
+                                    kv, n_max, ic, oc, _p(res))
+    return res
+
+
+def rule_conv_backward(d_out, feature, weight_oc_ic, rules, rule_size, tile_grid_shape):
+    """rule_conv.cu:577-597 -> (d_feature, d_weight[KV,iC,oC])."""
+    d_feature = rule_conv_d_feature(d_out, weight_oc_ic, rules, rule_size, tile_grid_shape,
+                                    feature.shape[0])
+    d_weight = rule_conv_d_weight(feature, d_out, rules, rule_size)
+    return d_feature, d_weight
+
+
+def rule_conv_i8(feature, weight, scale, rules, rule_size, out_nnz, return_acc=False):
+    feature = np.ascontiguousarray(feature, dtype=np.int8)
+    weight = np.ascontiguousarray(weight, dtype=np.int8)
+    scale = _f32(scale)
+    rules, rule_size = _i32(rules), _i32(rule_size)
+    ntile, kv, _, n_max = rules.shape
+    ic, oc = weight.shape[1], weight.shape[2]
+    out = np.empty((int(out_nnz), oc), np.int8)
+    acc = np.empty((int(out_nnz), oc), np.int32)
+    lib().orc_rule_conv_i8(_p(feature), _p(weight), _p(scale), _p(rules), _p(rule_size), ntile,
+                           kv, n_max, ic, oc, int(out_nnz), _p(acc), _p(out))
+    return (out, acc) if return_acc else out
