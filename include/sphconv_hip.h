@@ -1,0 +1,198 @@
+/*
+ * sphconv_hip.h -- C ABI of libsphconv_hip.so (gfx950 / MI355X).
+ *
+ * Drop-in boundary for the sparse-convolution hot path of reveriel/sphconv:
+ * the entry points below are what a binding of the reference's extension module
+ * `sphconv.sphconv_cuda` (src/sphconv/all.cpp:14-38) calls instead of the CUDA
+ * kernels.  Every pointer is a DEVICE pointer unless the comment says "host".
+ * The library never allocates, frees or synchronises: the caller provides all
+ * outputs and scratch, and every call only enqueues kernels on `stream`.
+ *
+ * Every function returns 0 on success or a negative sph_status; the message of
+ * the last failure on the calling thread is returned by sph_last_error().
+ *
+ * Data layout (same as the reference, tensor.py:33-102 / tensor.cu:78-127):
+ *   feature [rows, C]  row-major, element type given by sph_dtype
+ *   z_idx   [rows]     int32, S2 coordinate of each row
+ *   z_ptr   [B*S0*S1]  int32, INCLUSIVE prefix sum of per-column row counts in
+ *                      flattened (b,s0,s1) order
+ * Kernel offset index k = (k0*K1 + k1)*K2 + k2 (rules.cu:124-126); weight is
+ * [KV, iC, oC].  Input x pairs with output o_d = (x_d + pad_d - k_d) / stride_d
+ * iff divisible and 0 <= o_d < O_d (rules.cu:36-45); dilation is accepted and
+ * ignored exactly as the reference does (rules.cu:39-40).
+ *
+ * Rule book (this library's compact replacement of the reference's padded
+ * `rules [NTile,KV,2,tile_n_max]` tensor, rules.cu:364-366): the rows of the
+ * stationary side are cut into tiles of SPH_TILE_ROWS consecutive rows; the
+ * pairs of a tile are stored per kernel offset k, in ascending row order, in
+ * groups of SPH_GROUP slots padded with -1:
+ *   tile_ngrp [NT]              groups used by each tile
+ *   tile_koff [NT, KV+1] u16    first group of offset k inside the tile
+ *   grp_k     [NT*cap]          kernel offset of each group
+ *   grp_gather[NT*cap*16]       row on the gathered side (or -1)
+ *   grp_owner [NT*cap*16]       row on the stationary side (or -1)
+ * with NT = sph_book_tiles(rows) and cap = sph_book_cap(KV) groups per tile.
+ * A forward book is stationary on OUTPUT rows (gather = input row), a
+ * transposed book on INPUT rows (gather = output row; used by dgrad).
+ */
+#ifndef SPHCONV_HIP_H
+#define SPHCONV_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SPH_TILE_ROWS 128
+#define SPH_GROUP 16
+#define SPH_MAX_KV 128
+#define SPH_MAX_CHANNELS 256
+
+typedef enum sph_status {
+    SPH_OK = 0,
+    SPH_ERR_ARG = -1,         /* null pointer, bad size, bad enum                */
+    SPH_ERR_UNSUPPORTED = -2, /* channel count / kernel volume out of range      */
+    SPH_ERR_LAUNCH = -3       /* HIP reported an error at launch                 */
+} sph_status;
+
+typedef enum sph_dtype {
+    SPH_F32 = 0,  /* fp32 storage, fp32 accumulate                     */
+    SPH_F16 = 1,  /* fp16 storage, fp32 accumulate                     */
+    SPH_BF16 = 2, /* bf16 storage, fp32 accumulate                     */
+    SPH_I8 = 3    /* int8 storage, int32 accumulate, requantised store */
+} sph_dtype;
+
+/* Geometry of one convolution; argument meaning follows get_rules[_subm]
+ * (include/sphconv/rules.h:8-32): spatialShape, outSpatialShape, kernelSize,
+ * stride, padding, dilation, each ordered (S0,S1,S2). */
+typedef struct sph_geom {
+    int32_t B;
+    int32_t S[3];
+    int32_t O[3];
+    int32_t K[3];
+    int32_t stride[3];
+    int32_t pad[3];
+    int32_t dil[3];
+} sph_geom;
+
+typedef struct sph_book {
+    int32_t *tile_ngrp;
+    uint16_t *tile_koff;
+    int32_t *grp_k;
+    int32_t *grp_gather;
+    int32_t *grp_owner;
+    int32_t rows; /* rows on the stationary side */
+    int32_t KV;
+} sph_book;
+
+const char *sph_last_error(void);
+int sph_abi_version(void);
+
+/* Sizing helpers (host arithmetic only). */
+int sph_book_tiles(int rows);          /* NT = ceil(rows / SPH_TILE_ROWS)            */
+int sph_book_cap(int KV);              /* groups per tile = KV * SPH_TILE_ROWS / 16  */
+/* closed forms of the reference: rules.cu:21-34, conv.py:32-38 */
+int sph_tile_n_max(const sph_geom *g, int T0, int T1, int nnz);
+int sph_num_tiles(const sph_geom *g, int T0, int T1);
+
+/* ---- rule generation --------------------------------------------------- */
+
+/* Replaces get_rules_subm (rules.cu:326-390) and the pair half of get_rules
+ * (rules.cu:445-485): builds the rule book of one convolution.
+ *   transposed == 0: stationary side = output rows (oz_idx/oz_ptr over the O
+ *                    grid), gathered side = input rows (z_idx/z_ptr over S).
+ *   transposed == 1: stationary side = input rows, gathered side = output rows.
+ * For a submanifold convolution pass the input arrays as the output arrays and
+ * O == S.  `book.rows` must equal the stationary side's row count. */
+int sph_rules_build(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
+                    const int32_t *oz_idx, const int32_t *oz_ptr, int out_rows,
+                    const sph_geom *g, int transposed, const sph_book *book, void *stream);
+
+/* Replaces the output-coordinate half of get_rules (rules.cu:417-443, 461-462),
+ * in two steps because the caller must size oz_idx:
+ *  1. sph_outcoords_count: per-column output counts into oz_ptr (used as
+ *     scratch), block partial sums into block_sums [sph_outcoords_blocks(g)],
+ *     their exclusive scan in place, and the total in *total_dev (device int).
+ *  2. after reading *total_dev: sph_outcoords_fill writes the final oz_ptr
+ *     (inclusive scan) and oz_idx (ascending within a column). */
+int sph_outcoords_blocks(const sph_geom *g);
+int sph_outcoords_count(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
+                        const sph_geom *g, int32_t *oz_ptr, int32_t *block_sums,
+                        int32_t *total_dev, void *stream);
+int sph_outcoords_fill(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
+                       const sph_geom *g, const int32_t *block_sums, int32_t *oz_ptr,
+                       int32_t *oz_idx, int out_rows, void *stream);
+
+/* Conversions between the rule book and the reference's padded tensors
+ * `rules [NTile,KV,2,tile_n_max]`, `rule_size [NTile,KV]` (rules.cu:364-369).
+ * nbr is scratch of out_rows*KV int32 (forward) / in_rows*KV (transposed). */
+int sph_rules_to_padded_count(const sph_book *fwd_book, const int32_t *oz_ptr,
+                              const sph_geom *g, int T0, int T1, int32_t *nbr,
+                              int32_t *rule_size, void *stream);
+int sph_rules_to_padded_fill(const int32_t *oz_ptr, const sph_geom *g, int T0, int T1,
+                             const int32_t *nbr, int out_rows, int KV, int tile_n_max,
+                             int32_t *rules, void *stream);
+int sph_rules_from_padded(const int32_t *rules, const int32_t *rule_size, int ntile, int KV,
+                          int tile_n_max, int in_rows, int out_rows, int transposed,
+                          int32_t *nbr, const sph_book *book, void *stream);
+
+/* ---- convolution ------------------------------------------------------- */
+
+/* Bytes of the packed (MFMA fragment order) copy of a [KV, kdim, ndim] weight. */
+size_t sph_weight_packed_bytes(sph_dtype dt, int KV, int kdim, int ndim);
+/* Packs weight for the contraction  out[., n] += sum_kk in[., kk] * B[k][kk][n]
+ * where B[k][kk][n] = w[k*stride_k + kk*stride_kk + n*stride_n] (element strides). */
+int sph_weight_pack(sph_dtype dt, const void *w, int KV, int kdim, int ndim,
+                    long stride_k, long stride_kk, long stride_n, void *packed, void *stream);
+
+/* Optional epilogue applied to the accumulator before the store:
+ *   y = acc * scale[c] + shift[c]   (each pointer may be null: 1 / 0)
+ *   y = max(y, 0) if relu
+ * For SPH_I8, scale is required and the store is
+ *   q = clamp(rint((float)acc * scale[c]), -128, 127)      (shift, relu unused). */
+typedef struct sph_epilogue {
+    const float *scale;
+    const float *shift;
+    int32_t relu;
+} sph_epilogue;
+
+/* Replaces rule_conv (rule_conv.cu:286-336) and, with a transposed book and a
+ * weight packed from W[k]^T, rule_conv_d_feature (rule_conv.cu:520-575):
+ *   out[owner, :] = sum over the owner's pairs (k, gather) of
+ *                   feature[gather, :kdim] @ B[k]          (rows with no pair: 0)
+ * out has book->rows rows of ndim elements and is fully overwritten. */
+int sph_conv_apply(sph_dtype dt, const void *feature, int feature_rows, int kdim,
+                   const void *packed_w, int ndim, const sph_book *book,
+                   const sph_epilogue *epi, void *out, void *stream);
+
+/* Replaces rule_conv_d_weight (rule_conv.cu:469-518):
+ *   d_weight[k, ci, co] = sum over pairs (k, in, out) feature[in, ci] * d_out[out, co]
+ * from a FORWARD book.  partial is fp32 scratch of
+ * sph_wgrad_partial_elems(KV, iC, oC, rows) elements; the reduction over it is
+ * done in fp32 in a fixed order.  d_weight has the element type dt. */
+size_t sph_wgrad_partial_elems(int KV, int iC, int oC, int out_rows);
+int sph_conv_wgrad(sph_dtype dt, const void *feature, int in_rows, int iC, const void *d_out,
+                   int oC, const sph_book *fwd_book, float *partial, void *d_weight,
+                   void *stream);
+
+/* ---- tensor construction / densify (tensor.cu) ------------------------- */
+
+/* out[dst_row[n], :] = src[n, :] (dst_row null: identity) or, with gather != 0,
+ * out[n, :] = src[dst_row[n], :].  Rows of row_bytes bytes.  Replaces
+ * reorderFeatureKernel / reorderFeatureBackwardKernel (tensor.cu:39-76,130-145). */
+int sph_permute_rows(const void *src, const int32_t *index, int rows, int row_bytes,
+                     int gather, void *out, void *stream);
+/* Replaces to_dense / to_dense_backward (tensor.cu:222-309): dense is
+ * [B,S0,S1,S2,C]; only active cells are written (forward) / read (backward). */
+int sph_to_dense(const void *feature, const int32_t *z_idx, const int32_t *z_ptr, int rows,
+                 int ncol, int S2, int row_bytes, void *dense, void *stream);
+int sph_to_dense_backward(const void *d_dense, const int32_t *z_idx, const int32_t *z_ptr,
+                          int rows, int ncol, int S2, int row_bytes, void *d_feature,
+                          void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPHCONV_HIP_H */

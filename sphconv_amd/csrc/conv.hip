@@ -1,0 +1,534 @@
+// Gather-GEMM-scatter convolution for gfx950 (wave64, MFMA 16x16 tiles).
+//
+// Forward / dgrad (sph_conv_apply): one workgroup owns SPH_TILE_ROWS consecutive
+// owner rows; wave w owns owner columns [16w, 16w+16).  The tile's pairs arrive
+// as groups of 16 (one kernel offset per group).  Per group a wave gathers the 16
+// feature rows straight into MFMA A-fragments (16 B per lane), multiplies by the
+// pre-packed weight fragment of that offset and adds the 16x16 result into its
+// private columns of an LDS accumulator tile; the tile is written to HBM once,
+// with the epilogue fused.  No atomics, summation order fixed by the book.
+//
+// wgrad (sph_conv_wgrad): a workgroup owns (kernel offset, range of tiles),
+// transposes gathered rows through LDS so that the pair index becomes the MFMA
+// K dimension, keeps the [iC,oC] block in registers and writes one fp32 partial;
+// a second kernel sums the partials in a fixed order.
+#include "common.h"
+
+namespace {
+
+constexpr int R = SPH_TILE_ROWS;
+constexpr int kWave = 64;
+
+typedef int int4v __attribute__((ext_vector_type(4)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
+
+template <sph_dtype DT> struct Traits;
+template <> struct Traits<SPH_F32> {
+    typedef float elem;
+    typedef float4v acc4;
+    static constexpr int KW = 4; // elements per 16-byte fragment
+};
+template <> struct Traits<SPH_F16> {
+    typedef _Float16 elem;
+    typedef float4v acc4;
+    static constexpr int KW = 8;
+};
+template <> struct Traits<SPH_BF16> {
+    typedef __bf16 elem;
+    typedef float4v acc4;
+    static constexpr int KW = 8;
+};
+template <> struct Traits<SPH_I8> {
+    typedef int8_t elem;
+    typedef int4v acc4;
+    static constexpr int KW = 16;
+};
+
+// One "super step" consumes 64 bytes of every gathered row: lane l supplies the
+// 16 bytes at offset 16*(l/16) of row l%16 (A) / of column l%16 (B).  Any
+// assignment of K indices to lanes is valid as long as A and B agree.
+template <sph_dtype DT>
+__device__ __forceinline__ typename Traits<DT>::acc4 mfma_step(int4v a, int4v b, typename Traits<DT>::acc4 d);
+
+template <>
+__device__ __forceinline__ float4v mfma_step<SPH_F32>(int4v a, int4v b, float4v d)
+{
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        d = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[j]), __builtin_bit_cast(float, b[j]), d, 0, 0, 0);
+    return d;
+}
+template <>
+__device__ __forceinline__ float4v mfma_step<SPH_F16>(int4v a, int4v b, float4v d)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), d, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ float4v mfma_step<SPH_BF16>(int4v a, int4v b, float4v d)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, a), __builtin_bit_cast(bf8, b), d, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ int4v mfma_step<SPH_I8>(int4v a, int4v b, int4v d)
+{
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, d, 0, 0, 0);
+}
+
+// ---------------------------------------------------------------------------
+// Weight packing: packed[k][step][ntile][lane][KW] with
+//   kk = step*4*KW + KW*(lane/16) + j,  n = ntile*16 + lane%16,  zero padded.
+// ---------------------------------------------------------------------------
+template <sph_dtype DT>
+__global__ void pack_weight_kernel(const typename Traits<DT>::elem *w, int KV, int kdim, int ndim, long sk,
+                                   long skk, long sn, int nsteps, int ntn, typename Traits<DT>::elem *packed)
+{
+    constexpr int KW = Traits<DT>::KW;
+    long total = (long)KV * nsteps * ntn * kWave * KW;
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    int j = (int)(i % KW);
+    long t = i / KW;
+    int lane = (int)(t % kWave);
+    t /= kWave;
+    int nt = (int)(t % ntn);
+    t /= ntn;
+    int st = (int)(t % nsteps);
+    int k = (int)(t / nsteps);
+    int kk = st * 4 * KW + KW * (lane >> 4) + j;
+    int n = nt * 16 + (lane & 15);
+    typename Traits<DT>::elem v = (typename Traits<DT>::elem)0;
+    if (kk < kdim && n < ndim) v = w[k * sk + kk * skk + n * sn];
+    packed[i] = v;
+}
+
+struct ConvArgs {
+    const char *feat;
+    int feat_rows, kdim, row_bytes;
+    const char *wp;
+    int nsteps, ndim;
+    sph_book book;
+    int cap;
+    const float *scale, *shift;
+    int relu;
+    char *out;
+    int aligned_in, aligned_out;
+};
+
+template <sph_dtype DT>
+__device__ __forceinline__ int4v load_a_frag(const ConvArgs &a, int in_row, int st, int lane)
+{
+    typedef typename Traits<DT>::elem elem;
+    constexpr int KW = Traits<DT>::KW;
+    int4v f = {0, 0, 0, 0};
+    if ((unsigned)in_row >= (unsigned)a.feat_rows) return f;
+    const int byte_off = st * 64 + (lane >> 4) * 16;
+    const char *row = a.feat + (long)in_row * a.row_bytes;
+    if (a.aligned_in) {
+        if (byte_off < a.row_bytes) f = *(const int4v *)(row + byte_off);
+    } else {
+        union { int4v v; elem e[KW]; } u;
+        u.v = f;
+        const int c0 = byte_off / (int)sizeof(elem);
+#pragma unroll
+        for (int j = 0; j < KW; j++)
+            if (c0 + j < a.kdim) u.e[j] = ((const elem *)row)[c0 + j];
+        f = u.v;
+    }
+    return f;
+}
+
+template <sph_dtype DT>
+__device__ __forceinline__ float epilogue_value(const ConvArgs &a, uint32_t raw, int c)
+{
+    float v;
+    if (DT == SPH_I8)
+        v = (float)(int32_t)raw;
+    else
+        v = __builtin_bit_cast(float, raw);
+    if (a.scale) v = v * a.scale[c];
+    if (DT != SPH_I8) {
+        if (a.shift) v = v + a.shift[c];
+        if (a.relu) v = v > 0.f ? v : 0.f;
+    }
+    return v;
+}
+
+template <sph_dtype DT>
+__device__ __forceinline__ typename Traits<DT>::elem to_elem(float v)
+{
+    typedef typename Traits<DT>::elem elem;
+    if (DT == SPH_I8) {
+        float r = __builtin_rintf(v);
+        r = r < -128.f ? -128.f : (r > 127.f ? 127.f : r);
+        return (elem)(int)r;
+    }
+    return (elem)v;
+}
+
+template <sph_dtype DT, int NW>
+__global__ __launch_bounds__(NW * kWave) void conv_apply_kernel(ConvArgs a)
+{
+    typedef typename Traits<DT>::elem elem;
+    typedef typename Traits<DT>::acc4 acc4;
+    constexpr int LDW = NW * 16 + 4; // accumulator row stride in 32-bit words
+    extern __shared__ uint32_t s_acc[]; // [R][LDW]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int tile = blockIdx.x;
+    const int r0 = tile * R;
+    const int nrows = min(R, a.book.rows - r0);
+
+    // each wave clears and later updates only its own 16 columns
+    for (int i = lane; i < R * 16; i += kWave) s_acc[(i >> 4) * LDW + wave * 16 + (i & 15)] = 0u;
+
+    const int ngrp = a.book.tile_ngrp[tile];
+    const long gb0 = (long)tile * a.cap;
+    const int col = wave * 16 + (lane & 15);
+    for (int g = 0; g < ngrp; g++) {
+        const int k = a.book.grp_k[gb0 + g];
+        const long slot = (gb0 + g) * SPH_GROUP;
+        const int in_row = a.book.grp_gather[slot + (lane & 15)];
+        const int4v own = *(const int4v *)(a.book.grp_owner + slot + (lane >> 4) * 4);
+        acc4 d = {0, 0, 0, 0};
+        const char *wk = a.wp + ((long)k * a.nsteps * NW + wave) * (kWave * 16) + lane * 16;
+        for (int st = 0; st < a.nsteps; st++) {
+            int4v fa = load_a_frag<DT>(a, in_row, st, lane);
+            int4v fb = *(const int4v *)(wk + (long)st * NW * (kWave * 16));
+            d = mfma_step<DT>(fa, fb, d);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            int rl = own[r] - r0;
+            if ((unsigned)rl < (unsigned)nrows) {
+                uint32_t *p = &s_acc[rl * LDW + col];
+                if (DT == SPH_I8)
+                    *p = (uint32_t)((int32_t)*p + (int32_t)d[r]);
+                else
+                    *p = __builtin_bit_cast(uint32_t, __builtin_bit_cast(float, *p) + (float)d[r]);
+            }
+        }
+    }
+    __syncthreads();
+
+    // epilogue: LDS tile -> out rows [r0, r0+nrows), all ndim columns
+    elem *out = (elem *)a.out + (long)r0 * a.ndim;
+    constexpr int VE = 16 / (int)sizeof(elem);
+    if (a.aligned_out) {
+        const int cpr = a.ndim / VE; // 16-byte chunks per row
+        for (int i = tid; i < nrows * cpr; i += NW * kWave) {
+            int row = i / cpr, ch = i - row * cpr;
+            union { int4v v; elem e[VE]; } u;
+#pragma unroll
+            for (int j = 0; j < VE; j++)
+                u.e[j] = to_elem<DT>(epilogue_value<DT>(a, s_acc[row * LDW + ch * VE + j], ch * VE + j));
+            *(int4v *)(out + (long)row * a.ndim + ch * VE) = u.v;
+        }
+    } else {
+        for (int i = tid; i < nrows * a.ndim; i += NW * kWave) {
+            int row = i / a.ndim, c = i - row * a.ndim;
+            out[i] = to_elem<DT>(epilogue_value<DT>(a, s_acc[row * LDW + c], c));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// wgrad
+// ---------------------------------------------------------------------------
+struct WgradArgs {
+    const char *feat;
+    int in_rows, iC;
+    const char *dout;
+    int out_rows, oC;
+    sph_book book;
+    int cap, ntiles, nchunk;
+    float *partial;
+};
+
+constexpr int kWgThreads = 256;
+constexpr int kWgWaves = kWgThreads / kWave;
+constexpr int kMaxTilesPerWave = 16; // (128/16)^2 / 4 waves
+
+template <sph_dtype DT>
+__global__ __launch_bounds__(kWgThreads) void wgrad_kernel(WgradArgs a)
+{
+    typedef typename Traits<DT>::elem elem;
+    constexpr int KW = Traits<DT>::KW;
+    constexpr int PB = 4 * KW;            // pairs per batch = K of one super step
+    constexpr int LDP = PB + 16 / (int)sizeof(elem); // padded pair stride, keeps 16-byte alignment
+    extern __shared__ char s_raw[];
+    const int iCp = (a.iC + 15) & ~15, oCp = (a.oC + 15) & ~15;
+    elem *At = (elem *)s_raw;               // [iCp][LDP]
+    elem *Gt = At + (long)iCp * LDP;        // [oCp][LDP]
+    __shared__ int s_in[PB], s_out[PB];
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int KV = a.book.KV;
+    const int k = blockIdx.x / a.nchunk, chunk = blockIdx.x - k * a.nchunk;
+    const int tpc = (a.ntiles + a.nchunk - 1) / a.nchunk;
+    const int t0 = chunk * tpc, t1 = min(t0 + tpc, a.ntiles);
+    const int MI = iCp / 16, NI = oCp / 16, MT = MI * NI;
+
+    float4v acc[kMaxTilesPerWave];
+#pragma unroll
+    for (int j = 0; j < kMaxTilesPerWave; j++) acc[j] = float4v{0, 0, 0, 0};
+
+    for (int t = t0; t < t1; t++) {
+        const int g0 = a.book.tile_koff[(long)t * (KV + 1) + k];
+        const int g1 = a.book.tile_koff[(long)t * (KV + 1) + k + 1];
+        for (int gb = g0; gb < g1; gb += PB / SPH_GROUP) {
+            __syncthreads(); // previous batch fully consumed
+            if (tid < PB) {
+                int g = gb + tid / SPH_GROUP;
+                int vi = -1, vo = -1;
+                if (g < g1) {
+                    long slot = ((long)t * a.cap + g) * SPH_GROUP + (tid & (SPH_GROUP - 1));
+                    vi = a.book.grp_gather[slot];
+                    vo = a.book.grp_owner[slot];
+                }
+                if ((unsigned)vi >= (unsigned)a.in_rows || (unsigned)vo >= (unsigned)a.out_rows) vi = vo = -1;
+                s_in[tid] = vi;
+                s_out[tid] = vo;
+            }
+            __syncthreads();
+            for (int e = tid; e < PB * iCp; e += kWgThreads) {
+                int p = e / iCp, c = e - p * iCp;
+                int row = s_in[p];
+                elem v = (elem)0;
+                if (row >= 0 && c < a.iC) v = ((const elem *)a.feat)[(long)row * a.iC + c];
+                At[c * LDP + p] = v;
+            }
+            for (int e = tid; e < PB * oCp; e += kWgThreads) {
+                int p = e / oCp, c = e - p * oCp;
+                int row = s_out[p];
+                elem v = (elem)0;
+                if (row >= 0 && c < a.oC) v = ((const elem *)a.dout)[(long)row * a.oC + c];
+                Gt[c * LDP + p] = v;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < kMaxTilesPerWave; j++) {
+                int ti = wave + j * kWgWaves;
+                if (ti < MT) {
+                    int mi = ti / NI, ni = ti - mi * NI;
+                    int4v fa = *(const int4v *)(At + (mi * 16 + (lane & 15)) * LDP + (lane >> 4) * KW);
+                    int4v fb = *(const int4v *)(Gt + (ni * 16 + (lane & 15)) * LDP + (lane >> 4) * KW);
+                    acc[j] = mfma_step<DT>(fa, fb, acc[j]);
+                }
+            }
+        }
+    }
+    float *part = a.partial + ((long)k * a.nchunk + chunk) * a.iC * a.oC;
+#pragma unroll
+    for (int j = 0; j < kMaxTilesPerWave; j++) {
+        int ti = wave + j * kWgWaves;
+        if (ti < MT) {
+            int mi = ti / NI, ni = ti - mi * NI;
+            int co = ni * 16 + (lane & 15);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                int ci = mi * 16 + (lane >> 4) * 4 + r;
+                if (ci < a.iC && co < a.oC) part[(long)ci * a.oC + co] = acc[j][r];
+            }
+        }
+    }
+}
+
+template <sph_dtype DT>
+__global__ void wgrad_reduce_kernel(const float *partial, int KV, int nchunk, int per_k,
+                                    typename Traits<DT>::elem *dw)
+{
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (long)KV * per_k) return;
+    int k = (int)(i / per_k), e = (int)(i - (long)k * per_k);
+    const float *p = partial + (long)k * nchunk * per_k + e;
+    float s = 0.f;
+    for (int c = 0; c < nchunk; c++) s += p[(long)c * per_k];
+    dw[i] = (typename Traits<DT>::elem)s;
+}
+
+inline int elem_size(sph_dtype dt) { return dt == SPH_F32 ? 4 : (dt == SPH_I8 ? 1 : 2); }
+inline int frag_elems(sph_dtype dt) { return 16 / elem_size(dt); }
+inline int pad_waves(int ndim)
+{
+    int nt = sph_div_up(ndim, 16);
+    return nt <= 1 ? 1 : (nt <= 2 ? 2 : (nt <= 4 ? 4 : 8));
+}
+inline int num_steps(sph_dtype dt, int kdim) { return sph_div_up(kdim, 4 * frag_elems(dt)); }
+inline int wgrad_chunks(int ntiles) { return ntiles < 32 ? (ntiles < 1 ? 1 : ntiles) : 32; }
+
+template <typename K>
+inline int set_lds(K kernel, size_t bytes)
+{
+    if (bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e != hipSuccess) {
+            sph_set_error("hipFuncSetAttribute(%zu bytes of LDS): %s", bytes, hipGetErrorString(e));
+            return SPH_ERR_LAUNCH;
+        }
+    }
+    return SPH_OK;
+}
+
+template <sph_dtype DT, int NW>
+int launch_conv(const ConvArgs &a, int ntiles, hipStream_t st)
+{
+    size_t lds = (size_t)R * (NW * 16 + 4) * sizeof(uint32_t);
+    int rc = set_lds(conv_apply_kernel<DT, NW>, lds);
+    if (rc) return rc;
+    hipLaunchKernelGGL((conv_apply_kernel<DT, NW>), dim3(ntiles), dim3(NW * kWave), lds, st, a);
+    return sph_check_launch("sph_conv_apply");
+}
+
+template <sph_dtype DT>
+int launch_conv_nw(const ConvArgs &a, int nw, int ntiles, hipStream_t st)
+{
+    switch (nw) {
+    case 1: return launch_conv<DT, 1>(a, ntiles, st);
+    case 2: return launch_conv<DT, 2>(a, ntiles, st);
+    case 4: return launch_conv<DT, 4>(a, ntiles, st);
+    default: return launch_conv<DT, 8>(a, ntiles, st);
+    }
+}
+
+template <sph_dtype DT>
+int launch_pack(const void *w, int KV, int kdim, int ndim, long sk, long skk, long sn, void *packed, hipStream_t st)
+{
+    typedef typename Traits<DT>::elem elem;
+    int nsteps = num_steps(DT, kdim), ntn = pad_waves(ndim);
+    long total = (long)KV * nsteps * ntn * kWave * Traits<DT>::KW;
+    hipLaunchKernelGGL(pack_weight_kernel<DT>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                       (const elem *)w, KV, kdim, ndim, sk, skk, sn, nsteps, ntn, (elem *)packed);
+    return sph_check_launch("sph_weight_pack");
+}
+
+template <sph_dtype DT>
+int launch_wgrad(const WgradArgs &a, void *dw, hipStream_t st)
+{
+    typedef typename Traits<DT>::elem elem;
+    constexpr int LDP = 4 * Traits<DT>::KW + 16 / (int)sizeof(elem);
+    const int iCp = (a.iC + 15) & ~15, oCp = (a.oC + 15) & ~15;
+    size_t lds = (size_t)(iCp + oCp) * LDP * sizeof(elem);
+    const int KV = a.book.KV;
+    hipLaunchKernelGGL(wgrad_kernel<DT>, dim3(KV * a.nchunk), dim3(kWgThreads), lds, st, a);
+    int rc = sph_check_launch("sph_conv_wgrad");
+    if (rc) return rc;
+    int per_k = a.iC * a.oC;
+    long total = (long)KV * per_k;
+    hipLaunchKernelGGL(wgrad_reduce_kernel<DT>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                       a.partial, KV, a.nchunk, per_k, (elem *)dw);
+    return sph_check_launch("sph_conv_wgrad(reduce)");
+}
+
+inline int book_ok(const sph_book *b)
+{
+    return b && b->tile_ngrp && b->tile_koff && b->grp_k && b->grp_gather && b->grp_owner &&
+           b->rows >= 0 && b->KV > 0 && b->KV <= SPH_MAX_KV;
+}
+
+} // namespace
+
+SPH_EXPORT size_t sph_weight_packed_bytes(sph_dtype dt, int KV, int kdim, int ndim)
+{
+    if (KV <= 0 || kdim <= 0 || ndim <= 0 || (int)dt < 0 || (int)dt > 3) return 0;
+    return (size_t)KV * num_steps(dt, kdim) * pad_waves(ndim) * kWave * 16;
+}
+
+SPH_EXPORT int sph_weight_pack(sph_dtype dt, const void *w, int KV, int kdim, int ndim, long stride_k,
+                               long stride_kk, long stride_n, void *packed, void *stream)
+{
+    SPH_REQUIRE(w && packed, SPH_ERR_ARG, "sph_weight_pack: null pointer");
+    SPH_REQUIRE(KV > 0 && KV <= SPH_MAX_KV, SPH_ERR_UNSUPPORTED, "sph_weight_pack: kernel volume %d not in 1..%d", KV, SPH_MAX_KV);
+    SPH_REQUIRE(kdim > 0 && kdim <= SPH_MAX_CHANNELS, SPH_ERR_UNSUPPORTED,
+                "sph_weight_pack: %d input channels not in 1..%d", kdim, SPH_MAX_CHANNELS);
+    SPH_REQUIRE(ndim > 0 && ndim <= 128, SPH_ERR_UNSUPPORTED, "sph_weight_pack: %d output channels not in 1..128", ndim);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dt) {
+    case SPH_F32: return launch_pack<SPH_F32>(w, KV, kdim, ndim, stride_k, stride_kk, stride_n, packed, st);
+    case SPH_F16: return launch_pack<SPH_F16>(w, KV, kdim, ndim, stride_k, stride_kk, stride_n, packed, st);
+    case SPH_BF16: return launch_pack<SPH_BF16>(w, KV, kdim, ndim, stride_k, stride_kk, stride_n, packed, st);
+    case SPH_I8: return launch_pack<SPH_I8>(w, KV, kdim, ndim, stride_k, stride_kk, stride_n, packed, st);
+    }
+    sph_set_error("sph_weight_pack: unknown dtype %d", (int)dt);
+    return SPH_ERR_ARG;
+}
+
+SPH_EXPORT int sph_conv_apply(sph_dtype dt, const void *feature, int feature_rows, int kdim,
+                              const void *packed_w, int ndim, const sph_book *book,
+                              const sph_epilogue *epi, void *out, void *stream)
+{
+    SPH_REQUIRE(book_ok(book), SPH_ERR_ARG, "sph_conv_apply: bad book");
+    SPH_REQUIRE(packed_w && feature_rows >= 0 && (feature_rows == 0 || feature), SPH_ERR_ARG, "sph_conv_apply: null pointer");
+    SPH_REQUIRE((int)dt >= 0 && (int)dt <= 3, SPH_ERR_ARG, "sph_conv_apply: unknown dtype %d", (int)dt);
+    SPH_REQUIRE(kdim > 0 && kdim <= SPH_MAX_CHANNELS, SPH_ERR_UNSUPPORTED,
+                "sph_conv_apply: %d input channels not in 1..%d", kdim, SPH_MAX_CHANNELS);
+    SPH_REQUIRE(ndim > 0 && ndim <= 128, SPH_ERR_UNSUPPORTED, "sph_conv_apply: %d output channels not in 1..128", ndim);
+    SPH_REQUIRE(dt != SPH_I8 || (epi && epi->scale), SPH_ERR_ARG, "sph_conv_apply: int8 needs per-channel scales");
+    if (book->rows == 0) return SPH_OK;
+    SPH_REQUIRE(out, SPH_ERR_ARG, "sph_conv_apply: null output");
+    const int es = elem_size(dt);
+    ConvArgs a;
+    a.feat = (const char *)feature;
+    a.feat_rows = feature_rows;
+    a.kdim = kdim;
+    a.row_bytes = kdim * es;
+    a.wp = (const char *)packed_w;
+    a.nsteps = num_steps(dt, kdim);
+    a.ndim = ndim;
+    a.book = *book;
+    a.cap = sph_book_cap(book->KV);
+    a.scale = epi ? epi->scale : nullptr;
+    a.shift = epi ? epi->shift : nullptr;
+    a.relu = epi ? epi->relu : 0;
+    a.out = (char *)out;
+    a.aligned_in = (a.row_bytes % 16 == 0) && ((uintptr_t)feature % 16 == 0);
+    a.aligned_out = ((ndim * es) % 16 == 0) && ((uintptr_t)out % 16 == 0);
+    SPH_REQUIRE((uintptr_t)packed_w % 16 == 0, SPH_ERR_ARG, "sph_conv_apply: packed weight must be 16-byte aligned");
+    const int nw = pad_waves(ndim), nt = sph_book_tiles(book->rows);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dt) {
+    case SPH_F32: return launch_conv_nw<SPH_F32>(a, nw, nt, st);
+    case SPH_F16: return launch_conv_nw<SPH_F16>(a, nw, nt, st);
+    case SPH_BF16: return launch_conv_nw<SPH_BF16>(a, nw, nt, st);
+    default: return launch_conv_nw<SPH_I8>(a, nw, nt, st);
+    }
+}
+
+SPH_EXPORT size_t sph_wgrad_partial_elems(int KV, int iC, int oC, int out_rows)
+{
+    if (KV <= 0 || iC <= 0 || oC <= 0) return 0;
+    return (size_t)KV * wgrad_chunks(sph_book_tiles(out_rows)) * iC * oC;
+}
+
+SPH_EXPORT int sph_conv_wgrad(sph_dtype dt, const void *feature, int in_rows, int iC, const void *d_out,
+                              int oC, const sph_book *fwd_book, float *partial, void *d_weight, void *stream)
+{
+    SPH_REQUIRE(book_ok(fwd_book), SPH_ERR_ARG, "sph_conv_wgrad: bad book");
+    SPH_REQUIRE(partial && d_weight, SPH_ERR_ARG, "sph_conv_wgrad: null pointer");
+    SPH_REQUIRE(dt == SPH_F32 || dt == SPH_F16 || dt == SPH_BF16, SPH_ERR_UNSUPPORTED,
+                "sph_conv_wgrad: dtype %d has no weight gradient", (int)dt);
+    SPH_REQUIRE(iC > 0 && iC <= 128 && oC > 0 && oC <= 128, SPH_ERR_UNSUPPORTED,
+                "sph_conv_wgrad: channels %d->%d not in 1..128", iC, oC);
+    SPH_REQUIRE((in_rows == 0 || feature) && (fwd_book->rows == 0 || d_out), SPH_ERR_ARG, "sph_conv_wgrad: null pointer");
+    WgradArgs a;
+    a.feat = (const char *)feature;
+    a.in_rows = in_rows;
+    a.iC = iC;
+    a.dout = (const char *)d_out;
+    a.out_rows = fwd_book->rows;
+    a.oC = oC;
+    a.book = *fwd_book;
+    a.cap = sph_book_cap(fwd_book->KV);
+    a.ntiles = sph_book_tiles(fwd_book->rows);
+    a.nchunk = wgrad_chunks(a.ntiles);
+    a.partial = partial;
+    hipStream_t st = (hipStream_t)stream;
+    switch (dt) {
+    case SPH_F32: return launch_wgrad<SPH_F32>(a, d_weight, st);
+    case SPH_F16: return launch_wgrad<SPH_F16>(a, d_weight, st);
+    default: return launch_wgrad<SPH_BF16>(a, d_weight, st);
+    }
+}

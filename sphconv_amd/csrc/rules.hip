@@ -1,0 +1,659 @@
+// Rule (indice) generation for gfx950: output coordinates of a strided
+// convolution and the rule book of (kernel offset, gathered row, owner row)
+// triples, replacing the reference's dense [B,S0,S1,S2] position grid and
+// atomic counters (src/sphconv/rules.cu) by fiber joins, wave ballots and
+// prefix popcounts.  All kernels are integer and HBM/latency bound.
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWave = 64;
+constexpr int kWaves = kThreads / kWave;
+constexpr int R = SPH_TILE_ROWS;
+
+struct Grid3 {
+    int n0, n1, n2;
+};
+
+struct ConvParams {
+    int K0, K1, K2;
+    int s0, s1, s2;
+    int p0, p1, p2;
+};
+
+__device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+// Row range [start, end) of column c, clamped to [0, rows] so that inconsistent
+// caller data can never index outside the row arrays.
+__device__ __forceinline__ void fiber_range(const int32_t *ptr, int c, int rows, int &start, int &end)
+{
+    end = clampi(ptr[c], 0, rows);
+    start = c ? clampi(ptr[c - 1], 0, rows) : 0;
+    if (start > end) start = end;
+}
+
+// First column c in [0, n) with a[c] > target (n if none), found by all
+// kThreads threads of the block together: every round probes kThreads evenly
+// spaced positions of the remaining window, so 2-3 rounds cover any grid.
+// s_tmp: one LDS int.  Must be called by the whole block.
+__device__ int block_upper_bound(const int32_t *a, int n, int target, int *s_tmp)
+{
+    int lo = 0, hi = n;
+    const int tid = threadIdx.x;
+    while (hi > lo) {
+        int span = hi - lo;
+        int step = (span + kThreads - 1) / kThreads;
+        long pos = (long)lo + (long)tid * step;
+        bool pred = (pos < hi) ? (a[pos] > target) : true;
+        if (tid == 0) *s_tmp = kThreads;
+        __syncthreads();
+        if (pred) atomicMin(s_tmp, tid);
+        __syncthreads();
+        int f = *s_tmp;
+        __syncthreads();
+        if (f == kThreads) {
+            lo = lo + (kThreads - 1) * step + 1;
+        } else {
+            long nh = (long)lo + (long)f * step;
+            int new_hi = nh < hi ? (int)nh : hi;
+            int new_lo = (f == 0) ? lo : lo + (f - 1) * step + 1;
+            hi = new_hi;
+            lo = new_lo;
+        }
+    }
+    return lo;
+}
+
+// ---------------------------------------------------------------------------
+// Shared tail of the book builders: the block holds, in LDS, a table
+// nbr[row_local * KV + k] = gathered row or -1 for the `nrows` rows of tile
+// `tile` (first row r0).  Emits the tile's groups: per k, rows in ascending
+// order, 16 per group, last group padded with -1.
+// LDS scratch: s_cnt[KV], s_goff[KV + 1].
+// ---------------------------------------------------------------------------
+__device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int tile, int cap,
+                            int *s_cnt, int *s_goff, const sph_book &book)
+{
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+
+    for (int k = wave; k < KV; k += kWaves) {
+        int cnt = 0;
+        for (int h = 0; h < R; h += kWave) {
+            int row = h + lane;
+            int v = (row < nrows) ? nbr[row * KV + k] : -1;
+            cnt += __popcll(__ballot(v >= 0));
+        }
+        if (lane == 0) s_cnt[k] = cnt;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int g = 0;
+        for (int k = 0; k < KV; k++) {
+            s_goff[k] = g;
+            g += (s_cnt[k] + SPH_GROUP - 1) / SPH_GROUP;
+        }
+        s_goff[KV] = g;
+        book.tile_ngrp[tile] = g;
+    }
+    __syncthreads();
+
+    const long gbase_tile = (long)tile * cap;
+    for (int k = wave; k < KV; k += kWaves) {
+        const int cnt = s_cnt[k];
+        if (cnt == 0) continue;
+        const long slot0 = (gbase_tile + s_goff[k]) * SPH_GROUP;
+        int pos = 0;
+        for (int h = 0; h < R; h += kWave) {
+            int row = h + lane;
+            int v = (row < nrows) ? nbr[row * KV + k] : -1;
+            unsigned long long m = __ballot(v >= 0);
+            if (v >= 0) {
+                int my = pos + __popcll(m & ((1ull << lane) - 1ull));
+                book.grp_gather[slot0 + my] = v;
+                book.grp_owner[slot0 + my] = r0 + row;
+            }
+            pos += __popcll(m);
+        }
+        int padded = (cnt + SPH_GROUP - 1) / SPH_GROUP * SPH_GROUP;
+        if (lane < padded - cnt) {
+            book.grp_gather[slot0 + cnt + lane] = -1;
+            book.grp_owner[slot0 + cnt + lane] = -1;
+        }
+        int ng = padded / SPH_GROUP;
+        for (int g = lane; g < ng; g += kWave) book.grp_k[gbase_tile + s_goff[k] + g] = k;
+    }
+    for (int k = tid; k <= KV; k += kThreads)
+        book.tile_koff[(long)tile * (KV + 1) + k] = (uint16_t)s_goff[k];
+}
+
+// ---------------------------------------------------------------------------
+// Book builder by fiber join.  One block per tile of R stationary rows.
+//   1. map the tile's rows to their columns (block-wide search in q_ptr, then a
+//      walk over the covering columns);
+//   2. for every (row, k0, k1): locate the one column of the other grid that
+//      can pair with it and compare its fiber entries' S2 coordinate;
+//   3. emit_groups.
+// TRANSPOSED = false: stationary rows are outputs, x_d = o_d*s_d - p_d + k_d.
+// TRANSPOSED = true : stationary rows are inputs,  o_d = (x_d + p_d - k_d)/s_d.
+// ---------------------------------------------------------------------------
+struct BuildArgs {
+    const int32_t *q_idx, *q_ptr; // stationary side
+    const int32_t *p_idx, *p_ptr; // gathered side
+    int q_rows, p_rows;
+    int B;
+    Grid3 Q, P;
+    ConvParams cv;
+    int cap;
+    sph_book book;
+};
+
+template <bool TRANSPOSED>
+__global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
+{
+    extern __shared__ int32_t s_nbr[]; // [R * KV]
+    __shared__ int s_col[R];
+    __shared__ int s_b[R], s_c0[R], s_c1[R], s_z[R];
+    __shared__ int s_cnt[SPH_MAX_KV], s_goff[SPH_MAX_KV + 1];
+    __shared__ int s_tmp, s_flag;
+
+    const int tid = threadIdx.x;
+    const int tile = blockIdx.x;
+    const int KV = a.cv.K0 * a.cv.K1 * a.cv.K2;
+    const int K01 = a.cv.K0 * a.cv.K1;
+    const int r0 = tile * R;
+    const int r1 = min(r0 + R, a.q_rows);
+    const int nrows = r1 - r0;
+    const int q_ncol = a.B * a.Q.n0 * a.Q.n1;
+
+    for (int i = tid; i < R * KV; i += kThreads) s_nbr[i] = -1;
+    for (int i = tid; i < R; i += kThreads) s_col[i] = -1;
+
+    // 1. rows -> columns
+    int c_first = block_upper_bound(a.q_ptr, q_ncol, r0, &s_tmp);
+    bool done = (c_first >= q_ncol);
+    for (int cb = c_first; !done; cb += kThreads) {
+        int c = cb + tid;
+        int last = min(cb + kThreads - 1, q_ncol - 1);
+        if (c <= last) {
+            int s, e;
+            fiber_range(a.q_ptr, c, a.q_rows, s, e);
+            int lo = max(s, r0), hi = min(e, r1);
+            for (int r = lo; r < hi; r++) s_col[r - r0] = c;
+            if (c == last) s_flag = (e >= r1) || (last == q_ncol - 1);
+        }
+        __syncthreads();
+        done = s_flag != 0;
+        __syncthreads();
+    }
+    __syncthreads();
+    for (int i = tid; i < nrows; i += kThreads) {
+        int c = s_col[i];
+        if (c >= 0) {
+            int b = c / (a.Q.n0 * a.Q.n1);
+            int rem = c - b * (a.Q.n0 * a.Q.n1);
+            s_b[i] = b;
+            s_c0[i] = rem / a.Q.n1;
+            s_c1[i] = rem % a.Q.n1;
+            s_z[i] = a.q_idx[r0 + i];
+        }
+    }
+    __syncthreads();
+
+    // 2. join: item = (k01, row); consecutive lanes take consecutive rows
+    for (int it = tid; it < K01 * R; it += kThreads) {
+        int rl = it & (R - 1);
+        int k01 = it / R;
+        if (rl >= nrows || s_col[rl] < 0) continue;
+        int k0 = k01 / a.cv.K1, k1 = k01 - k0 * a.cv.K1;
+        int y0, y1;
+        if (!TRANSPOSED) {
+            y0 = s_c0[rl] * a.cv.s0 - a.cv.p0 + k0;
+            y1 = s_c1[rl] * a.cv.s1 - a.cv.p1 + k1;
+        } else {
+            int t0 = s_c0[rl] + a.cv.p0 - k0, t1 = s_c1[rl] + a.cv.p1 - k1;
+            if (t0 < 0 || t1 < 0 || t0 % a.cv.s0 || t1 % a.cv.s1) continue;
+            y0 = t0 / a.cv.s0;
+            y1 = t1 / a.cv.s1;
+        }
+        if (y0 < 0 || y0 >= a.P.n0 || y1 < 0 || y1 >= a.P.n1) continue;
+        int pc = (s_b[rl] * a.P.n0 + y0) * a.P.n1 + y1;
+        int ps, pe;
+        fiber_range(a.p_ptr, pc, a.p_rows, ps, pe);
+        const int z = s_z[rl];
+        for (int e = ps; e < pe; e++) {
+            int zz = a.p_idx[e];
+            int k2;
+            if (!TRANSPOSED)
+                k2 = zz - (z * a.cv.s2 - a.cv.p2); // zz is the input S2 coordinate
+            else
+                k2 = z + a.cv.p2 - zz * a.cv.s2;   // zz is the output S2 coordinate
+            if (k2 >= 0 && k2 < a.cv.K2) s_nbr[rl * KV + k01 * a.cv.K2 + k2] = e;
+        }
+    }
+    __syncthreads();
+
+    // 3. compaction
+    emit_groups(s_nbr, nrows, r0, KV, tile, a.cap, s_cnt, s_goff, a.book);
+}
+
+// Book builder from a global neighbour table nbr[rows, KV] (used when the rules
+// arrive in the reference's padded format).
+__global__ __launch_bounds__(kThreads) void book_from_nbr_kernel(const int32_t *nbr, int rows, int KV,
+                                                                 int cap, sph_book book)
+{
+    extern __shared__ int32_t s_nbr[];
+    __shared__ int s_cnt[SPH_MAX_KV], s_goff[SPH_MAX_KV + 1];
+    const int tile = blockIdx.x;
+    const int r0 = tile * R;
+    const int nrows = min(R, rows - r0);
+    for (int i = threadIdx.x; i < nrows * KV; i += kThreads) s_nbr[i] = nbr[(long)r0 * KV + i];
+    __syncthreads();
+    emit_groups(s_nbr, nrows, r0, KV, tile, cap, s_cnt, s_goff, book);
+}
+
+// ---------------------------------------------------------------------------
+// Output coordinates of a strided convolution.  One thread per output column:
+// the set of active S2 bins of the column is the union, over the K0*K1 input
+// columns that reach it, of the bins (z + p2 - k2)/s2.  Bins are collected as
+// 64-bit masks, 64 bins per pass (one pass when O2 <= 64).
+// ---------------------------------------------------------------------------
+struct OutArgs {
+    const int32_t *z_idx, *z_ptr;
+    int in_rows;
+    int B;
+    Grid3 S, O;
+    ConvParams cv;
+};
+
+__device__ unsigned long long column_mask(const OutArgs &a, int b, int o0, int o1, int chunk)
+{
+    unsigned long long mask = 0;
+    for (int k0 = 0; k0 < a.cv.K0; k0++) {
+        int x0 = o0 * a.cv.s0 - a.cv.p0 + k0;
+        if (x0 < 0 || x0 >= a.S.n0) continue;
+        for (int k1 = 0; k1 < a.cv.K1; k1++) {
+            int x1 = o1 * a.cv.s1 - a.cv.p1 + k1;
+            if (x1 < 0 || x1 >= a.S.n1) continue;
+            int pc = (b * a.S.n0 + x0) * a.S.n1 + x1;
+            int ps, pe;
+            fiber_range(a.z_ptr, pc, a.in_rows, ps, pe);
+            for (int e = ps; e < pe; e++) {
+                int z = a.z_idx[e];
+                for (int k2 = 0; k2 < a.cv.K2; k2++) {
+                    int t = z + a.cv.p2 - k2;
+                    if (t < 0 || t % a.cv.s2) continue;
+                    int o2 = t / a.cv.s2;
+                    if (o2 < a.O.n2 && (o2 >> 6) == chunk) mask |= 1ull << (o2 & 63);
+                }
+            }
+        }
+    }
+    return mask;
+}
+
+__global__ __launch_bounds__(kThreads) void outcoords_count_kernel(OutArgs a, int32_t *counts,
+                                                                   int32_t *block_sums)
+{
+    __shared__ int s_red[kWaves];
+    const int ncol = a.B * a.O.n0 * a.O.n1;
+    const int oc = blockIdx.x * kThreads + threadIdx.x;
+    int cnt = 0;
+    if (oc < ncol) {
+        int b = oc / (a.O.n0 * a.O.n1);
+        int rem = oc - b * (a.O.n0 * a.O.n1);
+        int o0 = rem / a.O.n1, o1 = rem % a.O.n1;
+        int nchunk = (a.O.n2 + 63) >> 6;
+        for (int ch = 0; ch < nchunk; ch++) cnt += __popcll(column_mask(a, b, o0, o1, ch));
+        counts[oc] = cnt;
+    }
+    // block sum
+    int v = cnt;
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_down(v, off, kWave);
+    if ((threadIdx.x & (kWave - 1)) == 0) s_red[threadIdx.x / kWave] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int s = 0;
+        for (int w = 0; w < kWaves; w++) s += s_red[w];
+        block_sums[blockIdx.x] = s;
+    }
+}
+
+// Exclusive scan of block_sums[n] in place by one block; total -> *total.
+__global__ __launch_bounds__(1024) void scan_block_sums_kernel(int32_t *block_sums, int n, int32_t *total)
+{
+    __shared__ int s_buf[1024];
+    __shared__ int s_carry;
+    if (threadIdx.x == 0) s_carry = 0;
+    __syncthreads();
+    for (int base = 0; base < n; base += 1024) {
+        int i = base + threadIdx.x;
+        int v = (i < n) ? block_sums[i] : 0;
+        s_buf[threadIdx.x] = v;
+        __syncthreads();
+        for (int off = 1; off < 1024; off <<= 1) {
+            int t = (threadIdx.x >= off) ? s_buf[threadIdx.x - off] : 0;
+            __syncthreads();
+            s_buf[threadIdx.x] += t;
+            __syncthreads();
+        }
+        int incl = s_buf[threadIdx.x];
+        int carry = s_carry;
+        if (i < n) block_sums[i] = carry + incl - v;
+        __syncthreads();
+        if (threadIdx.x == 1023) s_carry = carry + incl;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *total = s_carry;
+}
+
+__global__ __launch_bounds__(kThreads) void outcoords_fill_kernel(OutArgs a, const int32_t *block_offs,
+                                                                  int32_t *oz_ptr, int32_t *oz_idx,
+                                                                  int out_rows)
+{
+    __shared__ int s_buf[kThreads];
+    const int ncol = a.B * a.O.n0 * a.O.n1;
+    const int oc = blockIdx.x * kThreads + threadIdx.x;
+    int cnt = (oc < ncol) ? oz_ptr[oc] : 0; // per-column count left by the count kernel
+    s_buf[threadIdx.x] = cnt;
+    __syncthreads();
+    for (int off = 1; off < kThreads; off <<= 1) {
+        int t = (threadIdx.x >= off) ? s_buf[threadIdx.x - off] : 0;
+        __syncthreads();
+        s_buf[threadIdx.x] += t;
+        __syncthreads();
+    }
+    if (oc >= ncol) return;
+    int incl = block_offs[blockIdx.x] + s_buf[threadIdx.x];
+    oz_ptr[oc] = incl;
+    if (cnt == 0) return;
+    int pos = incl - cnt;
+    int b = oc / (a.O.n0 * a.O.n1);
+    int rem = oc - b * (a.O.n0 * a.O.n1);
+    int o0 = rem / a.O.n1, o1 = rem % a.O.n1;
+    int nchunk = (a.O.n2 + 63) >> 6;
+    for (int ch = 0; ch < nchunk; ch++) {
+        unsigned long long m = column_mask(a, b, o0, o1, ch);
+        while (m) {
+            int bit = __ffsll((long long)m) - 1;
+            if (pos < out_rows) oz_idx[pos] = ch * 64 + bit;
+            pos++;
+            m &= m - 1;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Conversions to / from the reference's padded rule tensors.
+// ---------------------------------------------------------------------------
+__global__ void fill_i32_kernel(int32_t *p, long n, int32_t v)
+{
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    long stride = (long)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) p[i] = v;
+}
+
+// nbr[owner * KV + k] = gather for every used slot of the book.
+__global__ void nbr_from_book_kernel(sph_book book, int cap, int ntiles, int32_t *nbr)
+{
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x; // slot index over ntiles*cap*16
+    long total = (long)ntiles * cap * SPH_GROUP;
+    if (i >= total) return;
+    long grp = i / SPH_GROUP;
+    int tile = (int)(grp / cap);
+    int g = (int)(grp - (long)tile * cap);
+    if (g >= book.tile_ngrp[tile]) return;
+    int owner = book.grp_owner[i];
+    if (owner < 0) return;
+    nbr[(long)owner * book.KV + book.grp_k[grp]] = book.grp_gather[i];
+}
+
+// One thread per (reference tile, k).  The tile covers output columns
+// [t0*T0, +T0) x [t1*T1, +T1) of every batch sample (debug_utils.h:37-42);
+// walking b, o0, o1, row ascending yields the list in ascending output row,
+// which for sorted fibers is also ascending input row.
+template <bool FILL>
+__global__ void padded_kernel(const int32_t *oz_ptr, int out_rows, int B, int O0, int O1, int T0, int T1,
+                              int KV, const int32_t *nbr, int tile_n_max, int32_t *rule_size,
+                              int32_t *rules)
+{
+    int tgw = (O1 + T1 - 1) / T1;
+    int ntile = ((O0 + T0 - 1) / T0) * tgw;
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (long)ntile * KV) return;
+    int t = (int)(i / KV), k = (int)(i - (long)t * KV);
+    int t0 = t / tgw, t1 = t - t0 * tgw;
+    int cnt = 0;
+    for (int b = 0; b < B; b++)
+        for (int o0 = t0 * T0; o0 < min((t0 + 1) * T0, O0); o0++)
+            for (int o1 = t1 * T1; o1 < min((t1 + 1) * T1, O1); o1++) {
+                int c = (b * O0 + o0) * O1 + o1;
+                int s, e;
+                fiber_range(oz_ptr, c, out_rows, s, e);
+                for (int j = s; j < e; j++) {
+                    int in = nbr[(long)j * KV + k];
+                    if (in < 0) continue;
+                    if (FILL && cnt < tile_n_max) {
+                        long base = ((long)t * KV + k) * 2 * tile_n_max;
+                        rules[base + cnt] = in;
+                        rules[base + tile_n_max + cnt] = j;
+                    }
+                    cnt++;
+                }
+            }
+    if (!FILL) rule_size[i] = cnt;
+}
+
+__global__ void nbr_from_padded_kernel(const int32_t *rules, const int32_t *rule_size, int ntile, int KV,
+                                       int tile_n_max, int in_rows, int out_rows, int transposed,
+                                       int32_t *nbr)
+{
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x; // over ntile*KV*tile_n_max
+    long total = (long)ntile * KV * tile_n_max;
+    if (i >= total) return;
+    long tk = i / tile_n_max;
+    int v = (int)(i - tk * tile_n_max);
+    int n = rule_size[tk];
+    if (v >= n) return;
+    int k = (int)(tk % KV);
+    int in = rules[tk * 2 * tile_n_max + v];
+    int out = rules[tk * 2 * tile_n_max + tile_n_max + v];
+    if (in < 0 || in >= in_rows || out < 0 || out >= out_rows) return;
+    if (!transposed)
+        nbr[(long)out * KV + k] = in;
+    else
+        nbr[(long)in * KV + k] = out;
+}
+
+inline ConvParams conv_params(const sph_geom *g)
+{
+    return ConvParams{g->K[0], g->K[1], g->K[2], g->stride[0], g->stride[1], g->stride[2],
+                      g->pad[0], g->pad[1], g->pad[2]};
+}
+
+inline int book_ok(const sph_book *b)
+{
+    return b && b->tile_ngrp && b->tile_koff && b->grp_k && b->grp_gather && b->grp_owner &&
+           b->rows >= 0 && b->KV > 0 && b->KV <= SPH_MAX_KV;
+}
+
+} // namespace
+
+// ---------------------------------------------------------------------------
+// Entry points
+// ---------------------------------------------------------------------------
+static thread_local char g_err[512] = "";
+
+void sph_set_error(const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+SPH_EXPORT const char *sph_last_error(void) { return g_err; }
+SPH_EXPORT int sph_abi_version(void) { return 1; }
+SPH_EXPORT int sph_book_tiles(int rows) { return rows <= 0 ? 0 : sph_div_up(rows, R); }
+SPH_EXPORT int sph_book_cap(int KV) { return KV * (R / SPH_GROUP); }
+
+SPH_EXPORT int sph_tile_n_max(const sph_geom *g, int T0, int T1, int nnz)
+{
+    SPH_REQUIRE(g && T0 > 0 && T1 > 0, SPH_ERR_ARG, "sph_tile_n_max: bad argument");
+    // rules.cu:21-34
+    int in0 = g->stride[0] * (T0 - 1) + g->K[0];
+    int in1 = g->stride[1] * (T1 - 1) + g->K[1];
+    double sparsity = (double)nnz / ((double)g->B * g->S[0] * g->S[1] * g->S[2]);
+    double size = (double)g->B * in0 * in1 * g->S[2] * sparsity * 2;
+    return (int)(size + 64) & ~15;
+}
+
+SPH_EXPORT int sph_num_tiles(const sph_geom *g, int T0, int T1)
+{
+    SPH_REQUIRE(g && T0 > 0 && T1 > 0, SPH_ERR_ARG, "sph_num_tiles: bad argument");
+    return sph_div_up(g->O[0], T0) * sph_div_up(g->O[1], T1);
+}
+
+SPH_EXPORT int sph_rules_build(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
+                               const int32_t *oz_idx, const int32_t *oz_ptr, int out_rows,
+                               const sph_geom *g, int transposed, const sph_book *book, void *stream)
+{
+    SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_rules_build: bad geometry (kernel volume <= %d)", SPH_MAX_KV);
+    SPH_REQUIRE(book_ok(book), SPH_ERR_ARG, "sph_rules_build: bad book");
+    SPH_REQUIRE(z_ptr && oz_ptr && in_rows >= 0 && out_rows >= 0, SPH_ERR_ARG, "sph_rules_build: bad argument");
+    SPH_REQUIRE((in_rows == 0 || z_idx) && (out_rows == 0 || oz_idx), SPH_ERR_ARG, "sph_rules_build: null index array");
+    const int KV = g->K[0] * g->K[1] * g->K[2];
+    SPH_REQUIRE(book->KV == KV, SPH_ERR_ARG, "sph_rules_build: book.KV %d != kernel volume %d", book->KV, KV);
+    SPH_REQUIRE(book->rows == (transposed ? in_rows : out_rows), SPH_ERR_ARG,
+                "sph_rules_build: book.rows %d does not match the stationary side", book->rows);
+    if (book->rows == 0) return SPH_OK;
+
+    BuildArgs a;
+    Grid3 S{g->S[0], g->S[1], g->S[2]}, O{g->O[0], g->O[1], g->O[2]};
+    if (!transposed) {
+        a.q_idx = oz_idx; a.q_ptr = oz_ptr; a.q_rows = out_rows; a.Q = O;
+        a.p_idx = z_idx;  a.p_ptr = z_ptr;  a.p_rows = in_rows;  a.P = S;
+    } else {
+        a.q_idx = z_idx;  a.q_ptr = z_ptr;  a.q_rows = in_rows;  a.Q = S;
+        a.p_idx = oz_idx; a.p_ptr = oz_ptr; a.p_rows = out_rows; a.P = O;
+    }
+    a.B = g->B;
+    a.cv = conv_params(g);
+    a.cap = sph_book_cap(KV);
+    a.book = *book;
+    const int nt = sph_book_tiles(book->rows);
+    const size_t lds = (size_t)R * KV * sizeof(int32_t);
+    hipStream_t st = (hipStream_t)stream;
+    if (!transposed)
+        hipLaunchKernelGGL(build_book_kernel<false>, dim3(nt), dim3(kThreads), lds, st, a);
+    else
+        hipLaunchKernelGGL(build_book_kernel<true>, dim3(nt), dim3(kThreads), lds, st, a);
+    return sph_check_launch("sph_rules_build");
+}
+
+SPH_EXPORT int sph_outcoords_blocks(const sph_geom *g)
+{
+    SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_blocks: bad geometry");
+    return sph_div_up(g->B * g->O[0] * g->O[1], kThreads);
+}
+
+static OutArgs out_args(const int32_t *z_idx, const int32_t *z_ptr, int in_rows, const sph_geom *g)
+{
+    OutArgs a;
+    a.z_idx = z_idx; a.z_ptr = z_ptr; a.in_rows = in_rows; a.B = g->B;
+    a.S = Grid3{g->S[0], g->S[1], g->S[2]};
+    a.O = Grid3{g->O[0], g->O[1], g->O[2]};
+    a.cv = conv_params(g);
+    return a;
+}
+
+SPH_EXPORT int sph_outcoords_count(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
+                                   const sph_geom *g, int32_t *oz_ptr, int32_t *block_sums,
+                                   int32_t *total_dev, void *stream)
+{
+    SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_count: bad geometry");
+    SPH_REQUIRE(z_ptr && oz_ptr && block_sums && total_dev && in_rows >= 0 && (in_rows == 0 || z_idx),
+                SPH_ERR_ARG, "sph_outcoords_count: null argument");
+    hipStream_t st = (hipStream_t)stream;
+    const int nb = sph_outcoords_blocks(g);
+    hipLaunchKernelGGL(outcoords_count_kernel, dim3(nb), dim3(kThreads), 0, st,
+                       out_args(z_idx, z_ptr, in_rows, g), oz_ptr, block_sums);
+    int rc = sph_check_launch("sph_outcoords_count");
+    if (rc) return rc;
+    hipLaunchKernelGGL(scan_block_sums_kernel, dim3(1), dim3(1024), 0, st, block_sums, nb, total_dev);
+    return sph_check_launch("sph_outcoords_count(scan)");
+}
+
+SPH_EXPORT int sph_outcoords_fill(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
+                                  const sph_geom *g, const int32_t *block_sums, int32_t *oz_ptr,
+                                  int32_t *oz_idx, int out_rows, void *stream)
+{
+    SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_fill: bad geometry");
+    SPH_REQUIRE(z_ptr && oz_ptr && block_sums && out_rows >= 0 && (out_rows == 0 || oz_idx) &&
+                    (in_rows == 0 || z_idx), SPH_ERR_ARG, "sph_outcoords_fill: null argument");
+    const int nb = sph_outcoords_blocks(g);
+    hipLaunchKernelGGL(outcoords_fill_kernel, dim3(nb), dim3(kThreads), 0, (hipStream_t)stream,
+                       out_args(z_idx, z_ptr, in_rows, g), block_sums, oz_ptr, oz_idx, out_rows);
+    return sph_check_launch("sph_outcoords_fill");
+}
+
+SPH_EXPORT int sph_rules_to_padded_count(const sph_book *fwd_book, const int32_t *oz_ptr,
+                                         const sph_geom *g, int T0, int T1, int32_t *nbr,
+                                         int32_t *rule_size, void *stream)
+{
+    SPH_REQUIRE(sph_geom_ok(g) && T0 > 0 && T1 > 0, SPH_ERR_ARG, "sph_rules_to_padded_count: bad geometry");
+    SPH_REQUIRE(book_ok(fwd_book) && oz_ptr && nbr && rule_size, SPH_ERR_ARG, "sph_rules_to_padded_count: null argument");
+    hipStream_t st = (hipStream_t)stream;
+    const int KV = fwd_book->KV, rows = fwd_book->rows;
+    const int nt = sph_book_tiles(rows), cap = sph_book_cap(KV);
+    long n = (long)rows * KV;
+    if (n > 0) {
+        hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)min((n + 255) / 256, 65535L)), dim3(256), 0, st, nbr, n, -1);
+        long slots = (long)nt * cap * SPH_GROUP;
+        hipLaunchKernelGGL(nbr_from_book_kernel, dim3((unsigned)((slots + 255) / 256)), dim3(256), 0, st,
+                           *fwd_book, cap, nt, nbr);
+    }
+    long ntk = (long)sph_num_tiles(g, T0, T1) * KV;
+    hipLaunchKernelGGL(padded_kernel<false>, dim3((unsigned)((ntk + 255) / 256)), dim3(256), 0, st, oz_ptr,
+                       rows, g->B, g->O[0], g->O[1], T0, T1, KV, nbr, 0, rule_size, (int32_t *)nullptr);
+    return sph_check_launch("sph_rules_to_padded_count");
+}
+
+SPH_EXPORT int sph_rules_to_padded_fill(const int32_t *oz_ptr, const sph_geom *g, int T0, int T1,
+                                        const int32_t *nbr, int out_rows, int KV, int tile_n_max,
+                                        int32_t *rules, void *stream)
+{
+    SPH_REQUIRE(sph_geom_ok(g) && T0 > 0 && T1 > 0 && tile_n_max > 0, SPH_ERR_ARG, "sph_rules_to_padded_fill: bad geometry");
+    SPH_REQUIRE(oz_ptr && nbr && rules && out_rows >= 0, SPH_ERR_ARG, "sph_rules_to_padded_fill: null argument");
+    hipStream_t st = (hipStream_t)stream;
+    long ntk = (long)sph_num_tiles(g, T0, T1) * KV;
+    long n = ntk * 2 * tile_n_max;
+    hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)min((n + 255) / 256, 65535L)), dim3(256), 0, st, rules, n, -1);
+    hipLaunchKernelGGL(padded_kernel<true>, dim3((unsigned)((ntk + 255) / 256)), dim3(256), 0, st, oz_ptr,
+                       out_rows, g->B, g->O[0], g->O[1], T0, T1, KV, nbr, tile_n_max, (int32_t *)nullptr, rules);
+    return sph_check_launch("sph_rules_to_padded_fill");
+}
+
+SPH_EXPORT int sph_rules_from_padded(const int32_t *rules, const int32_t *rule_size, int ntile, int KV,
+                                     int tile_n_max, int in_rows, int out_rows, int transposed,
+                                     int32_t *nbr, const sph_book *book, void *stream)
+{
+    SPH_REQUIRE(rules && rule_size && nbr && book_ok(book), SPH_ERR_ARG, "sph_rules_from_padded: null argument");
+    SPH_REQUIRE(ntile > 0 && KV > 0 && KV <= SPH_MAX_KV && tile_n_max > 0 && in_rows >= 0 && out_rows >= 0,
+                SPH_ERR_ARG, "sph_rules_from_padded: bad size");
+    const int rows = transposed ? in_rows : out_rows;
+    SPH_REQUIRE(book->rows == rows && book->KV == KV, SPH_ERR_ARG, "sph_rules_from_padded: book does not match");
+    if (rows == 0) return SPH_OK;
+    hipStream_t st = (hipStream_t)stream;
+    long n = (long)rows * KV;
+    hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)min((n + 255) / 256, 65535L)), dim3(256), 0, st, nbr, n, -1);
+    long total = (long)ntile * KV * tile_n_max;
+    hipLaunchKernelGGL(nbr_from_padded_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, rules,
+                       rule_size, ntile, KV, tile_n_max, in_rows, out_rows, transposed, nbr);
+    const int nt = sph_book_tiles(rows);
+    hipLaunchKernelGGL(book_from_nbr_kernel, dim3(nt), dim3(kThreads), (size_t)R * KV * sizeof(int32_t), st,
+                       nbr, rows, KV, sph_book_cap(KV), *book);
+    return sph_check_launch("sph_rules_from_padded");
+}

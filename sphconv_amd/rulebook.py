@@ -1,0 +1,210 @@
+"""Rule book: this package's compact form of the reference's rule tensors.
+
+The reference returns ``rules [NTile,KV,2,tile_n_max]`` padded with -1 plus
+``rule_size [NTile,KV]`` (src/sphconv/rules.cu:364-369): hundreds of megabytes of
+padding at LiDAR sizes.  A :class:`RuleBook` keeps the same pairs in the layout
+the HIP kernels consume (see ``include/sphconv_hip.h``) and materialises the
+padded tensors only when asked (:meth:`RuleBook.padded`).
+"""
+import ctypes as C
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import _lib as L
+
+
+class _Buffers:
+    """Device arrays of one book (forward or transposed)."""
+
+    def __init__(self, rows: int, kv: int, device):
+        lib = L.lib()
+        self.rows, self.kv = int(rows), int(kv)
+        self.ntiles = lib.sph_book_tiles(self.rows)
+        self.cap = lib.sph_book_cap(self.kv)
+        nt = max(self.ntiles, 1)
+        i32 = dict(dtype=torch.int32, device=device)
+        self.tile_ngrp = torch.empty(nt, **i32)
+        self.tile_koff = torch.empty((nt, self.kv + 1), dtype=torch.int16, device=device)
+        self.grp_k = torch.empty(nt * self.cap, **i32)
+        self.grp_gather = torch.empty(nt * self.cap * L.GROUP, **i32)
+        self.grp_owner = torch.empty(nt * self.cap * L.GROUP, **i32)
+
+    def struct(self) -> L.Book:
+        return L.Book(L.ptr(self.tile_ngrp), L.ptr(self.tile_koff), L.ptr(self.grp_k),
+                      L.ptr(self.grp_gather), L.ptr(self.grp_owner), self.rows, self.kv)
+
+    def num_pairs(self) -> int:
+        """Total pairs held (synchronises)."""
+        if self.ntiles == 0:
+            return 0
+        ng = self.tile_ngrp[:self.ntiles].long()
+        own = self.grp_owner.view(self.ntiles, self.cap * L.GROUP)
+        used = torch.arange(self.cap * L.GROUP, device=own.device)[None, :] < (ng * L.GROUP)[:, None]
+        return int(((own >= 0) & used).sum().item())
+
+
+class RuleBook:
+    """Pairs of one convolution geometry on one sparse tensor."""
+
+    def __init__(self, z_idx, z_ptr, oz_idx, oz_ptr, batch, in_shape, out_shape, kernel, stride,
+                 padding, dilation, subm):
+        self.z_idx, self.z_ptr = z_idx, z_ptr
+        self.oz_idx, self.oz_ptr = oz_idx, oz_ptr
+        self.batch = int(batch)
+        self.in_shape = [int(v) for v in in_shape]
+        self.out_shape = [int(v) for v in out_shape]
+        self.kernel = [int(v) for v in kernel]
+        self.stride = [int(v) for v in stride]
+        self.padding = [int(v) for v in padding]
+        self.dilation = [int(v) for v in dilation]
+        self.subm = bool(subm)
+        self.kv = self.kernel[0] * self.kernel[1] * self.kernel[2]
+        self.in_rows = int(z_idx.shape[0]) if z_idx is not None else 0
+        self.out_rows = int(oz_idx.shape[0]) if oz_idx is not None else 0
+        self.fwd: Optional[_Buffers] = None
+        self._bwd: Optional[_Buffers] = None
+        self._padded = {}
+        self._from_padded = None     # (rules, rule_size) when built from reference-format tensors
+
+    # -- construction -----------------------------------------------------
+    def geom(self) -> L.Geom:
+        return L.make_geom(self.batch, self.in_shape, self.out_shape, self.kernel, self.stride,
+                           self.padding, self.dilation)
+
+    def _build(self, transposed: bool) -> _Buffers:
+        rows = self.in_rows if transposed else self.out_rows
+        buf = _Buffers(rows, self.kv, self.z_ptr.device)
+        g, b = self.geom(), buf.struct()
+        L.check(L.lib().sph_rules_build(L.ptr(self.z_idx), L.ptr(self.z_ptr), self.in_rows,
+                                        L.ptr(self.oz_idx), L.ptr(self.oz_ptr), self.out_rows,
+                                        C.byref(g), int(transposed), C.byref(b), L.stream()))
+        return buf
+
+    @classmethod
+    def build_subm(cls, z_idx, z_ptr, batch, shape, kernel, padding=None,
+                   dilation=(1, 1, 1)) -> "RuleBook":
+        """Submanifold rules (replaces get_rules_subm, rules.cu:326-390): stride 1,
+        outputs are the inputs; ``padding`` defaults to K//2 (conv.py:210)."""
+        _check_index_tensors(z_idx, z_ptr, batch, shape)
+        pad = [int(k) // 2 for k in kernel] if padding is None else [int(v) for v in padding]
+        rb = cls(z_idx, z_ptr, z_idx, z_ptr, batch, shape, shape, kernel, (1, 1, 1), pad, dilation, True)
+        rb.fwd = rb._build(False)
+        return rb
+
+    @classmethod
+    def build(cls, z_idx, z_ptr, batch, in_shape, out_shape, kernel, stride, padding,
+              dilation=(1, 1, 1)) -> "RuleBook":
+        """Strided rules (replaces get_rules, rules.cu:405-486): output coordinates
+        (oz_ptr inclusive scan, oz_idx ascending per column) and pairs.  One
+        device->host read of the output row count, as in the reference (rules.cu:461)."""
+        _check_index_tensors(z_idx, z_ptr, batch, in_shape)
+        lib = L.lib()
+        dev = z_ptr.device
+        g = L.make_geom(batch, in_shape, out_shape, kernel, stride, padding, dilation)
+        if min(int(v) for v in out_shape) <= 0:
+            raise L.SphconvError("empty output grid %s" % (list(out_shape),))
+        nblk = lib.sph_outcoords_blocks(C.byref(g))
+        if nblk < 0:
+            L.check(nblk)
+        oz_ptr = torch.empty((int(batch), int(out_shape[0]), int(out_shape[1])), dtype=torch.int32, device=dev)
+        scratch = torch.empty(nblk + 1, dtype=torch.int32, device=dev)
+        total = scratch[nblk:]
+        n_in = int(z_idx.shape[0])
+        L.check(lib.sph_outcoords_count(L.ptr(z_idx), L.ptr(z_ptr), n_in, C.byref(g), L.ptr(oz_ptr),
+                                        L.ptr(scratch), total.data_ptr(), L.stream()))
+        out_rows = int(total.item())
+        oz_idx = torch.empty(out_rows, dtype=torch.int32, device=dev)
+        L.check(lib.sph_outcoords_fill(L.ptr(z_idx), L.ptr(z_ptr), n_in, C.byref(g), L.ptr(scratch),
+                                       L.ptr(oz_ptr), L.ptr(oz_idx), out_rows, L.stream()))
+        rb = cls(z_idx, z_ptr, oz_idx, oz_ptr, batch, in_shape, out_shape, kernel, stride, padding,
+                 dilation, False)
+        rb.fwd = rb._build(False)
+        return rb
+
+    @classmethod
+    def from_padded(cls, rules, rule_size, in_rows: int, out_rows: int) -> "RuleBook":
+        """Book from the reference's padded tensors (any tile size)."""
+        if rules.dim() != 4 or rules.shape[2] != 2 or rule_size.dim() != 2 \
+                or rule_size.shape[0] != rules.shape[0] or rule_size.shape[1] != rules.shape[1]:
+            raise L.SphconvError("rules must be [NTile,KV,2,n] and rule_size [NTile,KV], got %s, %s"
+                                 % (tuple(rules.shape), tuple(rule_size.shape)))
+        if rules.dtype != torch.int32 or rule_size.dtype != torch.int32:
+            raise L.SphconvError("rules and rule_size must be int32")
+        rb = cls.__new__(cls)
+        rb.z_idx = rb.z_ptr = rb.oz_idx = rb.oz_ptr = None
+        rb.batch = 0
+        rb.in_shape = rb.out_shape = rb.kernel = rb.stride = rb.padding = rb.dilation = None
+        rb.subm = False
+        rb.kv = int(rules.shape[1])
+        rb.in_rows, rb.out_rows = int(in_rows), int(out_rows)
+        rb._bwd = None
+        rb._padded = {}
+        rb._from_padded = (rules.contiguous(), rule_size.contiguous())
+        rb.fwd = rb._convert(False)
+        return rb
+
+    def _convert(self, transposed: bool) -> _Buffers:
+        rules, rule_size = self._from_padded
+        rows = self.in_rows if transposed else self.out_rows
+        buf = _Buffers(rows, self.kv, rules.device)
+        nbr = torch.empty(max(rows, 1) * self.kv, dtype=torch.int32, device=rules.device)
+        b = buf.struct()
+        L.check(L.lib().sph_rules_from_padded(L.ptr(rules), L.ptr(rule_size), int(rules.shape[0]),
+                                              self.kv, int(rules.shape[3]), self.in_rows,
+                                              self.out_rows, int(transposed), L.ptr(nbr),
+                                              C.byref(b), L.stream()))
+        return buf
+
+    # -- views ------------------------------------------------------------
+    def transposed(self) -> _Buffers:
+        """Book stationary on input rows (what dgrad gathers through)."""
+        if self._bwd is None:
+            self._bwd = self._convert(True) if self._from_padded is not None else self._build(True)
+        return self._bwd
+
+    def num_pairs(self) -> int:
+        return self.fwd.num_pairs()
+
+    def padded(self, tile_size: Sequence[int] = (2, 2)):
+        """-> (rules [NTile,KV,2,tile_n_max], rule_size [NTile,KV]) in the reference's
+        format, lists in ascending output row.  ``tile_n_max`` is the reference's
+        heuristic (rules.cu:21-28) raised, if needed, to the longest list so that no
+        pair is dropped (the reference drops them, rules.cu:301-308)."""
+        if self._from_padded is not None:
+            return self._from_padded
+        key = (int(tile_size[0]), int(tile_size[1]))
+        if key not in self._padded:
+            lib = L.lib()
+            g, b = self.geom(), self.fwd.struct()
+            dev = self.z_ptr.device
+            ntile = lib.sph_num_tiles(C.byref(g), *key)
+            nbr = torch.empty(max(self.out_rows, 1) * self.kv, dtype=torch.int32, device=dev)
+            rule_size = torch.empty((ntile, self.kv), dtype=torch.int32, device=dev)
+            L.check(lib.sph_rules_to_padded_count(C.byref(b), L.ptr(self.oz_ptr), C.byref(g), key[0],
+                                                  key[1], L.ptr(nbr), L.ptr(rule_size), L.stream()))
+            n_max = lib.sph_tile_n_max(C.byref(g), key[0], key[1], self.in_rows)
+            longest = int(rule_size.max().item()) if rule_size.numel() else 0
+            n_max = max(n_max, (longest + 15) & ~15, 16)
+            rules = torch.empty((ntile, self.kv, 2, n_max), dtype=torch.int32, device=dev)
+            L.check(lib.sph_rules_to_padded_fill(L.ptr(self.oz_ptr), C.byref(g), key[0], key[1],
+                                                 L.ptr(nbr), self.out_rows, self.kv, n_max,
+                                                 L.ptr(rules), L.stream()))
+            self._padded[key] = (rules, rule_size)
+        return self._padded[key]
+
+    def tile_grid_shape(self, tile_size: Sequence[int] = (2, 2)) -> List[int]:
+        """conv.py:32-38"""
+        return [-(-self.out_shape[0] // int(tile_size[0])), -(-self.out_shape[1] // int(tile_size[1]))]
+
+
+def _check_index_tensors(z_idx, z_ptr, batch, shape):
+    if z_idx.dtype != torch.int32 or z_ptr.dtype != torch.int32:
+        raise L.SphconvError("z_idx and z_ptr must be int32")
+    if z_idx.dim() != 1:
+        raise L.SphconvError("z_idx must be [NNZ]")
+    want = (int(batch), int(shape[0]), int(shape[1]))
+    if tuple(z_ptr.shape) != want:
+        raise L.SphconvError("z_ptr must be [B,S0,S1] = %s, got %s" % (want, tuple(z_ptr.shape)))
+    if not (z_idx.is_contiguous() and z_ptr.is_contiguous()):
+        raise L.SphconvError("z_idx and z_ptr must be contiguous")

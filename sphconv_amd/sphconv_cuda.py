@@ -1,0 +1,248 @@
+"""The reference's extension module, re-implemented over ``libsphconv_hip.so``.
+
+Same function names, argument order and return values as the pybind11 module
+``sphconv.sphconv_cuda`` (src/sphconv/all.cpp:18-31), so code written against the
+reference (``from sphconv.sphconv_cuda import get_rules, rule_conv ...``) runs
+unchanged with ``sphconv_amd.sphconv_cuda``.  Differences, all additive:
+
+* fibers come out of ``init_tensor`` sorted by S2 and rule lists sorted by row
+  (the reference leaves both in atomic-race order);
+* ``rules`` may be a :class:`~sphconv_amd.rulebook.RuleBook` (what
+  :func:`get_rulebook` / :func:`get_rulebook_subm` return) wherever the reference
+  takes its padded tensor -- the fast path that never materialises the padding;
+* float16 / bfloat16 features (fp32 accumulate) and int8 (:func:`rule_conv_int8`);
+* bad arguments raise ``SphconvError`` / ``ValueError`` instead of aborting.
+"""
+import ctypes as C
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import _lib as L
+from .rulebook import RuleBook
+
+__version__ = "hip-gfx950"
+
+def _packed_weight(weight: torch.Tensor, transpose: bool) -> torch.Tensor:
+    """weight [KV, a, b] -> fragment-ordered copy for the contraction over ``a``
+    (``transpose``: over ``b``, i.e. with W[k]^T).  Packed on every call: the
+    weight may have been updated in place since the last one."""
+    lib = L.lib()
+    w = weight.detach()
+    if not w.is_contiguous():
+        w = w.contiguous()
+    kv, a, b = w.shape
+    kdim, ndim = (b, a) if transpose else (a, b)
+    skk, sn = (1, b) if transpose else (b, 1)
+    dt = L.dtype_code(w.dtype)
+    nbytes = lib.sph_weight_packed_bytes(dt, kv, kdim, ndim)
+    if nbytes == 0:
+        raise L.SphconvError("cannot pack weight of shape %s" % (tuple(w.shape),))
+    packed = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+    L.check(lib.sph_weight_pack(dt, L.ptr(w), kv, kdim, ndim, a * b, skk, sn, L.ptr(packed), L.stream()))
+    return packed
+
+
+def _as_book(rules, rule_size, in_rows: int, out_rows: int) -> RuleBook:
+    if isinstance(rules, RuleBook):
+        return rules
+    return RuleBook.from_padded(rules, rule_size, in_rows, out_rows)
+
+
+def _apply(feature, packed, kdim, ndim, buffers, scale=None, shift=None, relu=False, out_dtype=None):
+    feature = feature.contiguous()
+    out = torch.empty((buffers.rows, ndim), dtype=out_dtype or feature.dtype, device=feature.device)
+    epi = L.Epilogue(L.ptr(scale), L.ptr(shift), int(bool(relu)))
+    b = buffers.struct()
+    L.check(L.lib().sph_conv_apply(L.dtype_code(feature.dtype), L.ptr(feature), int(feature.shape[0]),
+                                   int(kdim), L.ptr(packed), int(ndim), C.byref(b), C.byref(epi),
+                                   L.ptr(out), L.stream()))
+    return out
+
+
+# ---- tensor.h ---------------------------------------------------------------
+
+def init_tensor(feature: torch.Tensor, indicesBZYX: torch.Tensor, batchSize: int,
+                spatialShape: Sequence[int]) -> List[torch.Tensor]:
+    """tensor.cu:78-127 -> [outFeature, zIndices, zPtr, permutation].  Rows of a
+    fiber are ordered by ascending S2 (one legal order of the reference's output).
+    Sorting and the prefix sum use torch device ops; the row move is a HIP kernel."""
+    if indicesBZYX.dtype != torch.int32 or indicesBZYX.dim() != 2 or indicesBZYX.shape[1] != 4:
+        raise ValueError("indices must be int32 [NNZ,4] (b,s0,s1,s2)")
+    if feature.dim() != 2 or feature.shape[0] != indicesBZYX.shape[0]:
+        raise ValueError("feature must be [NNZ,C]")
+    S0, S1, S2 = (int(v) for v in spatialShape)
+    B = int(batchSize)
+    n = feature.shape[0]
+    dev = feature.device
+    idx = indicesBZYX.long()
+    if n:
+        lim = torch.tensor([B, S0, S1, S2], device=dev)
+        if bool(((idx < 0) | (idx >= lim)).any()):
+            raise ValueError("voxel coordinate outside batch/spatial shape %s" % ([B, S0, S1, S2],))
+    key = ((idx[:, 0] * S0 + idx[:, 1]) * S1 + idx[:, 2]) * S2 + idx[:, 3]
+    skey, order = torch.sort(key)
+    if n > 1 and bool((skey[1:] == skey[:-1]).any()):
+        raise ValueError("duplicate voxel coordinates")
+    z_idx = (skey % S2).to(torch.int32)
+    counts = torch.bincount(torch.div(skey, S2, rounding_mode="floor"), minlength=B * S0 * S1)
+    z_ptr = torch.cumsum(counts, 0).to(torch.int32).view(B, S0, S1)
+    permutation = torch.empty(n, dtype=torch.int32, device=dev)
+    permutation[order] = torch.arange(n, dtype=torch.int32, device=dev)
+    feature = feature.contiguous()
+    out = torch.empty_like(feature)
+    L.check(L.lib().sph_permute_rows(L.ptr(feature), L.ptr(permutation), n,
+                                     feature.shape[1] * feature.element_size(), 0, L.ptr(out), L.stream()))
+    return [out, z_idx, z_ptr, permutation]
+
+
+def init_tensor_backward(d_featureOut: torch.Tensor, permutation: torch.Tensor) -> torch.Tensor:
+    """tensor.cu:147-162: d_feature[n] = d_featureOut[permutation[n]]."""
+    d = d_featureOut.contiguous()
+    out = torch.empty_like(d)
+    L.check(L.lib().sph_permute_rows(L.ptr(d), L.ptr(permutation.contiguous()), d.shape[0],
+                                     d.shape[1] * d.element_size(), 1, L.ptr(out), L.stream()))
+    return out
+
+
+def to_dense(feature: torch.Tensor, zIndices: torch.Tensor, zPtr: torch.Tensor, D: int,
+             out: torch.Tensor) -> torch.Tensor:
+    """tensor.cu:222-264: writes active cells of ``out`` [B,S0,S1,S2,C] and returns it."""
+    feature = feature.contiguous()
+    if out.dim() != 5 or out.shape[4] != feature.shape[1] or out.dtype != feature.dtype:
+        raise ValueError("out must be [B,S0,S1,S2,C] of the feature's dtype")
+    ncol = zPtr.numel()
+    if out.shape[0] * out.shape[1] * out.shape[2] != ncol or out.shape[3] != int(D):
+        raise ValueError("out shape %s does not match z_ptr %s and D=%d"
+                         % (tuple(out.shape), tuple(zPtr.shape), D))
+    L.check(L.lib().sph_to_dense(L.ptr(feature), L.ptr(zIndices), L.ptr(zPtr), feature.shape[0], ncol,
+                                 int(D), feature.shape[1] * feature.element_size(), L.ptr(out), L.stream()))
+    return out
+
+
+def to_dense_backward(d_featureOut: torch.Tensor, zIndices: torch.Tensor, zPtr: torch.Tensor) -> torch.Tensor:
+    """tensor.cu:266-309: gathers [B,S0,S1,S2,C] gradients at the active cells."""
+    d = d_featureOut.contiguous()
+    n, c = zIndices.shape[0], d.shape[4]
+    out = torch.zeros((n, c), dtype=d.dtype, device=d.device)
+    L.check(L.lib().sph_to_dense_backward(L.ptr(d), L.ptr(zIndices), L.ptr(zPtr), n, zPtr.numel(),
+                                          d.shape[3], c * d.element_size(), L.ptr(out), L.stream()))
+    return out
+
+
+# ---- rules.h ----------------------------------------------------------------
+
+def get_rulebook_subm(zIndices, zPtr, batchSize, spatialShape, outSpatialShape, kernelSize, stride,
+                      padding, dilation, tileSize=None) -> RuleBook:
+    """Fast form of :func:`get_rules_subm`: the compact rule book only."""
+    if any(int(s) != 1 for s in stride):
+        raise L.SphconvError("submanifold convolution needs stride 1, got %s" % (list(stride),))
+    if list(map(int, spatialShape)) != list(map(int, outSpatialShape)):
+        raise L.SphconvError("submanifold convolution keeps the spatial shape")
+    return RuleBook.build_subm(zIndices, zPtr, batchSize, spatialShape, kernelSize, padding, dilation)
+
+
+def get_rulebook(zIndices, zPtr, batchSize, spatialShape, outSpatialShape, kernelSize, stride,
+                 padding, dilation, tileSize=None) -> RuleBook:
+    """Fast form of :func:`get_rules`."""
+    return RuleBook.build(zIndices, zPtr, batchSize, spatialShape, outSpatialShape, kernelSize,
+                          stride, padding, dilation)
+
+
+def get_rules_subm(zIndices, zPtr, batchSize, spatialShape, outSpatialShape, kernelSize, stride,
+                   padding, dilation, tileSize) -> List[torch.Tensor]:
+    """rules.cu:326-390 -> [zIndices, zPtr, rules, ruleSize] (the input index
+    tensors are returned as they are, rules.cu:389)."""
+    book = get_rulebook_subm(zIndices, zPtr, batchSize, spatialShape, outSpatialShape, kernelSize,
+                             stride, padding, dilation)
+    rules, rule_size = book.padded(tileSize)
+    return [zIndices, zPtr, rules, rule_size]
+
+
+def get_rules(zIndices, zPtr, batchSize, spatialShape, outSpatialShape, kernelSize, stride,
+              padding, dilation, tileSize) -> List[torch.Tensor]:
+    """rules.cu:405-486 -> [ozIndices, ozPtr, rules, ruleSize]."""
+    book = get_rulebook(zIndices, zPtr, batchSize, spatialShape, outSpatialShape, kernelSize, stride,
+                        padding, dilation)
+    rules, rule_size = book.padded(tileSize)
+    return [book.oz_idx, book.oz_ptr, rules, rule_size]
+
+
+# ---- rule_conv.h ------------------------------------------------------------
+
+def _check_conv_args(feature, weight):
+    if feature.dim() != 2 or weight.dim() != 3 or feature.shape[1] != weight.shape[1]:
+        raise L.SphconvError("feature [N,iC] / weight [KV,iC,oC] mismatch: %s vs %s"
+                             % (tuple(feature.shape), tuple(weight.shape)))
+    if weight.dtype != feature.dtype:
+        weight = weight.to(feature.dtype)
+    return weight
+
+
+def rule_conv(feature: torch.Tensor, weight: torch.Tensor, rules, ruleSize, outNNZ: int,
+              scale: Optional[torch.Tensor] = None, shift: Optional[torch.Tensor] = None,
+              relu: bool = False) -> torch.Tensor:
+    """rule_conv.cu:286-336: out[j] = sum over pairs (k,i,j) feature[i] @ weight[k].
+    ``scale``/``shift`` (fp32 [oC]) and ``relu`` fuse y = relu(acc*scale + shift)
+    into the store (no reference counterpart; default off)."""
+    weight = _check_conv_args(feature, weight)
+    book = _as_book(rules, ruleSize, feature.shape[0], int(outNNZ))
+    if book.out_rows != int(outNNZ) or book.kv != weight.shape[0]:
+        raise L.SphconvError("rules hold %d output rows / %d offsets, call says %d / %d"
+                             % (book.out_rows, book.kv, int(outNNZ), weight.shape[0]))
+    packed = _packed_weight(weight, False)
+    return _apply(feature, packed, weight.shape[1], weight.shape[2], book.fwd, scale, shift, relu)
+
+
+def rule_conv_int8(feature: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, rules, ruleSize,
+                   outNNZ: int) -> torch.Tensor:
+    """int8 x int8 -> int32 accumulate -> int8 with per-output-channel scales:
+    q = clamp(rint(float(acc) * scale[oc]), -128, 127), round half to even."""
+    if feature.dtype != torch.int8 or weight.dtype != torch.int8:
+        raise L.SphconvError("rule_conv_int8 needs int8 feature and weight")
+    _check_conv_args(feature, weight)
+    book = _as_book(rules, ruleSize, feature.shape[0], int(outNNZ))
+    packed = _packed_weight(weight, False)
+    return _apply(feature, packed, weight.shape[1], weight.shape[2], book.fwd,
+                  scale.to(torch.float32).contiguous())
+
+
+def rule_conv_d_feature(feature: torch.Tensor, weight: torch.Tensor, rules, ruleSize,
+                        tile_grid_shape, outNNZ: int) -> torch.Tensor:
+    """rule_conv.cu:520-575.  ``feature`` is d_out [outRows,oC], ``weight`` the
+    forward weight permuted to [KV,oC,iC] (functional.py:73), ``outNNZ`` the number
+    of input rows; returns d_feature [outNNZ,iC]."""
+    weight = _check_conv_args(feature, weight)
+    book = _as_book(rules, ruleSize, int(outNNZ), feature.shape[0])
+    packed = _packed_weight(weight, False)
+    return _apply(feature, packed, weight.shape[1], weight.shape[2], book.transposed())
+
+
+def rule_conv_d_weight(feature: torch.Tensor, d_featureOut: torch.Tensor, rules, ruleSize) -> torch.Tensor:
+    """rule_conv.cu:469-518 -> d_weight [KV,iC,oC], reduced in fp32."""
+    book = _as_book(rules, ruleSize, feature.shape[0], d_featureOut.shape[0])
+    feature = feature.contiguous()
+    d_out = d_featureOut.contiguous()
+    if d_out.dtype != feature.dtype:
+        d_out = d_out.to(feature.dtype)
+    lib = L.lib()
+    ic, oc = feature.shape[1], d_out.shape[1]
+    n = lib.sph_wgrad_partial_elems(book.kv, ic, oc, book.out_rows)
+    partial = torch.empty(max(n, 1), dtype=torch.float32, device=feature.device)
+    dw = torch.empty((book.kv, ic, oc), dtype=feature.dtype, device=feature.device)
+    b = book.fwd.struct()
+    L.check(lib.sph_conv_wgrad(L.dtype_code(feature.dtype), L.ptr(feature), feature.shape[0], ic,
+                               L.ptr(d_out), oc, C.byref(b), L.ptr(partial), L.ptr(dw), L.stream()))
+    return dw
+
+
+def rule_conv_backward(d_featureOut: torch.Tensor, feature: torch.Tensor, weight: torch.Tensor, rules,
+                       ruleSize, tile_grid_shape) -> List[torch.Tensor]:
+    """rule_conv.cu:577-597 -> [d_feature, d_weight]; ``weight`` is [KV,oC,iC]."""
+    book = _as_book(rules, ruleSize, feature.shape[0], d_featureOut.shape[0])
+    d_out = d_featureOut.contiguous()
+    if d_out.dtype != feature.dtype:
+        d_out = d_out.to(feature.dtype)
+    d_feature = rule_conv_d_feature(d_out, weight, book, None, tile_grid_shape, feature.shape[0])
+    d_weight = rule_conv_d_weight(feature, d_out, book, None)
+    return [d_feature, d_weight]

@@ -1,0 +1,277 @@
+"""GPU parity of the convolution kernels (forward, dgrad, wgrad, int8) against
+the CPU oracle, through the C ABI.
+
+Tolerances (stated by the task): fp32 rtol 1e-5 (atol 1e-5 for sums that cancel);
+fp16/bf16 storage with fp32 accumulate rtol 1e-2 / atol 1e-3 against a float64
+evaluation on the rounded inputs, scaled by the row's absolute-sum magnitude
+where outputs cancel; int8 bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+import gpu_helpers as G
+from oracle import oracle as O
+from sphconv_amd import sphconv_cuda as ext
+from sphconv_amd.synth import make_config
+
+pytestmark = pytest.mark.gpu
+CASES = H.load_ref_cases()
+
+
+def _conv_calls():
+    out = []
+    for tc in CASES:
+        if tc["file"] != "test/test_conv.py":
+            continue
+        for c in tc["calls"]:
+            out.append(pytest.param(tc["tensors"][c["coords"]], c["args"],
+                                    id="test_conv.py:%d" % c["line"]))
+    return out
+
+
+def _weights(rng, kv, ic, oc):
+    return (rng.standard_normal((kv, ic, oc)) / np.sqrt(kv * ic)).astype(np.float32)
+
+
+def _oracle_fwd(case, feat, w):
+    oz_idx, _, rules, rule_size, _ = case["oracle"]
+    return O.rule_conv(feat, w, rules, rule_size, oz_idx.shape[0])
+
+
+@pytest.mark.parametrize("coords,args", _conv_calls())
+def test_fp32_forward_reference_lists(coords, args):
+    a = args
+    subm = a.get("subm", False)
+    idx = H.dup_with_batch_idx(coords, a["batch_size"])
+    case = G.build_case(idx, a["batch_size"], a["spatial_shape_DWH"], a["kernel_size"], a["stride"],
+                        a["padding"], subm)
+    rng = np.random.default_rng(1)
+    ic, oc, kv = a["in_channels"], a["out_channels"], int(np.prod(a["kernel_size"]))
+    feat = rng.standard_normal((case["sidx"].shape[0], ic)).astype(np.float32)
+    w = _weights(rng, kv, ic, oc)
+    book = case["book"]
+    out = ext.rule_conv(G.t(feat), G.t(w), book, None, book.out_rows).cpu().numpy()
+    np.testing.assert_allclose(out, _oracle_fwd(case, feat, w), rtol=1e-5, atol=1e-5)
+    # the reference-format entry: padded rules + rule_size through the same call
+    rules, rule_size = book.padded((2, 2))
+    out2 = ext.rule_conv(G.t(feat), G.t(w), rules, rule_size, book.out_rows).cpu().numpy()
+    assert np.array_equal(out, out2)
+    # and against torch's dense conv3d in float64
+    dense = H.dense_from_rows(feat, case["sidx"], case["B"], case["shape"])
+    y = H.dense_conv(dense, w.reshape(*a["kernel_size"], ic, oc), case["stride"], case["padding"], case["oshape"])
+    out_coords, _, _ = H.brute_rules(case["sidx"], case["B"], case["shape"], a["kernel_size"],
+                                     case["stride"], case["padding"], subm)
+    np.testing.assert_allclose(out, H.gather_rows(y, out_coords).numpy(), rtol=1e-4, atol=1e-5)
+
+
+def _random_case(seed, subm, kernel=(3, 3, 3), stride=(2, 2, 2), padding=(1, 1, 1), B=2,
+                 shape=(11, 40, 24), p=0.25):
+    rng = np.random.default_rng(seed)
+    occ = rng.random((B, *shape)) < p
+    idx = np.argwhere(occ).astype(np.int32)
+    return G.build_case(idx, B, list(shape), list(kernel), list(stride), list(padding), subm)
+
+
+CHANNELS = [(1, 1), (3, 5), (4, 4), (5, 8), (16, 16), (17, 33), (32, 32), (32, 64), (64, 64), (64, 128),
+            (128, 64), (100, 20)]
+
+
+@pytest.mark.parametrize("ic,oc", CHANNELS)
+@pytest.mark.parametrize("subm", [True, False])
+def test_fp32_forward_channels(ic, oc, subm):
+    case = _random_case(ic * 131 + oc, subm)
+    rng = np.random.default_rng(2)
+    feat = rng.standard_normal((case["sidx"].shape[0], ic)).astype(np.float32)
+    w = _weights(rng, 27, ic, oc)
+    book = case["book"]
+    out = ext.rule_conv(G.t(feat), G.t(w), book, None, book.out_rows).cpu().numpy()
+    np.testing.assert_allclose(out, _oracle_fwd(case, feat, w), rtol=1e-5, atol=1e-5)
+
+
+def _f64_pair_sum(case, feat64, w64, transposed=False):
+    """sum over oracle pairs in float64 (definition), vectorised per (k)."""
+    oz_idx, _, rules, rule_size, _ = case["oracle"]
+    tri = G.oracle_triples(rules, rule_size)
+    if not transposed:
+        out = np.zeros((oz_idx.shape[0], w64.shape[2]))
+        absacc = np.zeros_like(out)
+        for k in np.unique(tri[:, 0]):
+            s = tri[tri[:, 0] == k]
+            out[s[:, 2]] += feat64[s[:, 1]] @ w64[k]
+            absacc[s[:, 2]] += np.abs(feat64[s[:, 1]]) @ np.abs(w64[k])
+    else:
+        out = np.zeros((case["sidx"].shape[0], w64.shape[1]))
+        absacc = np.zeros_like(out)
+        for k in np.unique(tri[:, 0]):
+            s = tri[tri[:, 0] == k]
+            out[s[:, 1]] += feat64[s[:, 2]] @ w64[k].T
+            absacc[s[:, 1]] += np.abs(feat64[s[:, 2]]) @ np.abs(w64[k]).T
+    return out, absacc
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("ic,oc", [(4, 4), (16, 16), (32, 32), (32, 64), (64, 64), (24, 40), (128, 128)])
+@pytest.mark.parametrize("subm", [True, False])
+def test_half_forward(dtype, ic, oc, subm):
+    case = _random_case(7 + ic + oc, subm)
+    rng = np.random.default_rng(3)
+    feat = torch.tensor(rng.standard_normal((case["sidx"].shape[0], ic)), dtype=torch.float32).to(dtype)
+    w = torch.tensor(_weights(rng, 27, ic, oc)).to(dtype)
+    book = case["book"]
+    out = ext.rule_conv(feat.to(G.DEV), w.to(G.DEV), book, None, book.out_rows)
+    assert out.dtype == dtype
+    ref, mag = _f64_pair_sum(case, feat.double().numpy(), w.double().numpy())
+    # output rounding: half an ulp of the storage type relative to the value
+    eps = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
+    err = np.abs(out.double().cpu().numpy() - ref)
+    assert (err <= 1e-3 + 1e-2 * np.abs(ref)).all()
+    assert (err <= 1e-6 + 2 * eps * np.abs(ref) + 1e-5 * mag).all()     # fp32 accumulate, one rounding
+
+
+@pytest.mark.parametrize("ic,oc", [(16, 8), (64, 64), (20, 36), (128, 128)])
+@pytest.mark.parametrize("subm", [True, False])
+def test_int8_forward_exact(ic, oc, subm):
+    case = _random_case(11 + ic, subm)
+    rng = np.random.default_rng(4)
+    n = case["sidx"].shape[0]
+    f8 = rng.integers(-128, 128, (n, ic), dtype=np.int8)
+    w8 = rng.integers(-128, 128, (27, ic, oc), dtype=np.int8)
+    scale = ((rng.random(oc) + 0.5) / (40.0 * ic)).astype(np.float32)
+    oz_idx, _, rules, rule_size, _ = case["oracle"]
+    want = O.rule_conv_i8(f8, w8, scale, rules, rule_size, oz_idx.shape[0])
+    book = case["book"]
+    got = ext.rule_conv_int8(G.t(f8), G.t(w8), G.t(scale), book, None, book.out_rows).cpu().numpy()
+    assert got.dtype == np.int8
+    assert np.array_equal(got, want)
+    assert want.min() == -128 and want.max() == 127 and (np.abs(want) < 100).mean() > 0.3
+
+
+@pytest.mark.parametrize("ic,oc", [(4, 4), (16, 16), (32, 64), (64, 64), (9, 21)])
+@pytest.mark.parametrize("subm,kernel,stride,padding", [
+    (True, (3, 3, 3), (1, 1, 1), (1, 1, 1)),
+    (False, (3, 3, 3), (2, 2, 2), (1, 1, 1)),
+    (False, (2, 2, 1), (1, 1, 1), (0, 0, 0)),
+])
+def test_fp32_backward(ic, oc, subm, kernel, stride, padding):
+    case = _random_case(21 + ic, subm, kernel, stride, padding)
+    rng = np.random.default_rng(5)
+    kv = int(np.prod(kernel))
+    n, m = case["sidx"].shape[0], case["oracle"][0].shape[0]
+    feat = rng.standard_normal((n, ic)).astype(np.float32)
+    w = _weights(rng, kv, ic, oc)
+    g = rng.standard_normal((m, oc)).astype(np.float32)
+    w_perm = np.ascontiguousarray(w.transpose(0, 2, 1))
+    _, _, rules, rule_size, _ = case["oracle"]
+    tgs = [-(-case["oshape"][0] // 2), -(-case["oshape"][1] // 2)]
+    d_feat_o, d_w_o = O.rule_conv_backward(g, feat, w_perm, rules, rule_size, tgs)
+    book = case["book"]
+    # reference entry point: weight pre-permuted to [KV,oC,iC]
+    d_feat, d_w = ext.rule_conv_backward(G.t(g), G.t(feat), G.t(w_perm), book, None, tgs)
+    np.testing.assert_allclose(d_feat.cpu().numpy(), d_feat_o, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(d_w.cpu().numpy(), d_w_o, rtol=1e-4, atol=1e-4)
+    # same through padded rules
+    pr, ps = book.padded((2, 2))
+    d_feat2, d_w2 = ext.rule_conv_backward(G.t(g), G.t(feat), G.t(w_perm), pr, ps, tgs)
+    assert np.array_equal(d_feat2.cpu().numpy(), d_feat.cpu().numpy())
+    assert np.array_equal(d_w2.cpu().numpy(), d_w.cpu().numpy())
+    # float64 definition
+    ref, _ = _f64_pair_sum(case, g.astype(np.float64), w.astype(np.float64), transposed=True)
+    np.testing.assert_allclose(d_feat.cpu().numpy(), ref, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_half_backward(dtype):
+    case = _random_case(31, True, p=0.3)
+    rng = np.random.default_rng(6)
+    n = case["sidx"].shape[0]
+    feat = torch.tensor(rng.standard_normal((n, 64)), dtype=torch.float32).to(dtype)
+    w = torch.tensor(_weights(rng, 27, 64, 64)).to(dtype)
+    g = torch.tensor(rng.standard_normal((n, 64)), dtype=torch.float32).to(dtype)
+    book = case["book"]
+    d_feat, d_w = ext.rule_conv_backward(g.to(G.DEV), feat.to(G.DEV),
+                                         w.permute(0, 2, 1).contiguous().to(G.DEV), book, None, [1, 1])
+    ref, _ = _f64_pair_sum(case, g.double().numpy(), w.double().numpy(), transposed=True)
+    err = np.abs(d_feat.double().cpu().numpy() - ref)
+    assert (err <= 1e-3 + 1e-2 * np.abs(ref)).all()
+    tri = G.oracle_triples(case["oracle"][2], case["oracle"][3])
+    dw_ref = np.zeros((27, 64, 64))
+    f64, g64 = feat.double().numpy(), g.double().numpy()
+    for k in range(27):
+        s = tri[tri[:, 0] == k]
+        dw_ref[k] = f64[s[:, 1]].T @ g64[s[:, 2]]
+    err = np.abs(d_w.double().cpu().numpy() - dw_ref)
+    assert (err <= 1e-3 + 1e-2 * np.abs(dw_ref) + 2e-3 * np.sqrt(n)).all()
+
+
+def test_fused_epilogue_scale_shift_relu():
+    case = _random_case(41, True)
+    rng = np.random.default_rng(7)
+    n = case["sidx"].shape[0]
+    feat = rng.standard_normal((n, 16)).astype(np.float32)
+    w = _weights(rng, 27, 16, 32)
+    scale = (rng.random(32) + 0.5).astype(np.float32)
+    shift = rng.standard_normal(32).astype(np.float32)
+    book = case["book"]
+    plain = ext.rule_conv(G.t(feat), G.t(w), book, None, n)
+    fused = ext.rule_conv(G.t(feat), G.t(w), book, None, n, scale=G.t(scale), shift=G.t(shift), relu=True)
+    want = torch.relu(plain * G.t(scale) + G.t(shift))
+    torch.testing.assert_close(fused, want, rtol=1e-6, atol=1e-6)
+
+
+def test_stable_case_extreme_weights():
+    """Reference test_stable.py:15-194: 74 voxels, stride 2, 64->64, extreme weights."""
+    tc = [c for c in CASES if c["file"] == "test/test_stable.py"][0]
+    coords = np.array(tc["tensors"]["indices_bzyx"], np.int32)
+    case = G.build_case(coords, 1, [6, 6, 20], [3, 3, 3], [2, 2, 2], [1, 1, 1], False)
+    raw = np.full((coords.shape[0], 64), 100.0, np.float32)
+    raw[0, :] = 8.0
+    raw[3, :] = 16.0
+    _, order = H.canonical_rows(coords)
+    feat = raw[order]
+    w = (np.random.default_rng(0).standard_normal((3, 3, 3, 64, 64)) / 2).astype(np.float32)
+    w[1] = 8.0
+    w[-1] = 100.0
+    w[1, 2, 0, :5, :] = 1 / 64
+    book = case["book"]
+    out = ext.rule_conv(G.t(feat), G.t(w.reshape(27, 64, 64)), book, None, book.out_rows).cpu().numpy()
+    want = _oracle_fwd(case, feat, w.reshape(27, 64, 64))
+    np.testing.assert_allclose(out, want, rtol=1e-5, atol=1e-2)
+    # run-to-run determinism (reference test_stable.py repeats the call)
+    for _ in range(3):
+        again = ext.rule_conv(G.t(feat), G.t(w.reshape(27, 64, 64)), book, None, book.out_rows).cpu().numpy()
+        assert np.array_equal(again, out)
+
+
+def test_config1_full_size_fp32():
+    """BASELINE config 1 at full size against the oracle (C, fp32)."""
+    d = make_config(1, seed=0)
+    shape, B = d["spatial_shape"], d["batch"]
+    rng = np.random.default_rng(0)
+    n = d["z_idx"].shape[0]
+    feat = rng.standard_normal((n, 16)).astype(np.float32)
+    w = _weights(rng, 27, 16, 16)
+    from sphconv_amd.rulebook import RuleBook
+    book = RuleBook.build_subm(G.t(d["z_idx"]), G.t(d["z_ptr"]), B, shape, [3, 3, 3])
+    out = ext.rule_conv(G.t(feat), G.t(w), book, None, n).cpu().numpy()
+    _, _, rules, rule_size, dropped = O.get_rules_subm(d["z_idx"], d["z_ptr"], B, shape, shape, [3, 3, 3],
+                                                       [1, 1, 1], [1, 1, 1], n_max=256)
+    assert dropped == 0
+    want = O.rule_conv(feat, w, rules, rule_size, n)
+    np.testing.assert_allclose(out, want, rtol=1e-5, atol=1e-5)
+
+
+def test_errors_are_reported_not_fatal():
+    from sphconv_amd import SphconvError
+    case = _random_case(51, True)
+    n = case["sidx"].shape[0]
+    book = case["book"]
+    with pytest.raises(SphconvError):
+        ext.rule_conv(torch.zeros((n, 8), device=G.DEV), torch.zeros((27, 8, 200), device=G.DEV), book, None, n)
+    with pytest.raises(SphconvError):
+        ext.rule_conv(torch.zeros((n, 8), device=G.DEV), torch.zeros((27, 9, 8), device=G.DEV), book, None, n)
+    with pytest.raises(SphconvError):
+        ext.rule_conv(torch.zeros((n, 8), device=G.DEV, dtype=torch.float64),
+                      torch.zeros((27, 8, 8), device=G.DEV, dtype=torch.float64), book, None, n)
+    with pytest.raises(SphconvError):
+        ext.rule_conv(torch.zeros((n, 8)), torch.zeros((27, 8, 8)), book, None, n)   # CPU tensors

@@ -1,0 +1,118 @@
+"""Module-level GPU tests: the reference's Python API (SparseConvTensor, Conv3d /
+SubMConv3d, Sequential, RangeVoxel, autograd) against torch's dense conv3d."""
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+import gpu_helpers as G
+import sphconv_amd as sphconv
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(seed, B, shape, C, p=0.2, dtype=torch.float32):
+    rng = np.random.default_rng(seed)
+    occ = rng.random((B, *shape)) < p
+    idx = np.argwhere(occ).astype(np.int32)
+    idx = idx[rng.permutation(idx.shape[0])]
+    feat = rng.standard_normal((idx.shape[0], C)).astype(np.float32)
+    return idx, feat
+
+
+def test_dense_roundtrip_and_grads():
+    """Reference test_grad.py:144-185: scaling dense cells by 2 and 3 gives grads 2 and 3."""
+    idx, feat = _inputs(0, 2, [5, 6, 7], 3)
+    f = G.t(feat).requires_grad_(True)
+    x = sphconv.SparseConvTensor(f, [5, 6, 7], 2, indices=G.t(idx))
+    dense = x.dense()
+    assert list(dense.shape) == [2, 3, 5, 6, 7]
+    want = H.dense_from_rows(feat, idx, 2, [5, 6, 7], torch.float32)
+    assert torch.equal(dense.detach().cpu(), want)
+    scale = torch.ones_like(dense)
+    scale[0] = 2.0
+    scale[1] = 3.0
+    (dense * scale).sum().backward()
+    g = f.grad.cpu().numpy()
+    assert np.array_equal(g[idx[:, 0] == 0], np.full_like(g[idx[:, 0] == 0], 2.0))
+    assert np.array_equal(g[idx[:, 0] == 1], np.full_like(g[idx[:, 0] == 1], 3.0))
+
+
+@pytest.mark.parametrize("subm,stride,padding", [(True, 1, 1), (False, 2, 1), (False, 1, 0)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_conv_module_matches_dense_autograd(subm, stride, padding, dtype):
+    B, shape, ic, oc = 2, [8, 12, 10], 8, 16
+    idx, feat = _inputs(1, B, shape, ic)
+    cls = sphconv.SubMConv3d if subm else sphconv.SparseConv3d
+    conv = cls(ic, oc, 3, stride=stride, padding=padding, bias=False).to(G.DEV).to(dtype)
+    f = G.t(feat).to(dtype).requires_grad_(True)
+    x = sphconv.SparseConvTensor(f, shape, B, indices=G.t(idx))
+    y = conv(x)
+    dense_y = y.dense()
+    # dense reference in float64 on the same (rounded) values
+    w64 = conv.weight.detach().double().cpu().requires_grad_(True)
+    f64 = f.detach().double().cpu().requires_grad_(True)
+    c = torch.as_tensor(idx, dtype=torch.long)
+    d_in = torch.zeros((B, *shape, ic), dtype=torch.float64).index_put((c[:, 0], c[:, 1], c[:, 2], c[:, 3]), f64)
+    ref = torch.nn.functional.conv3d(d_in.permute(0, 4, 1, 2, 3), w64.permute(4, 3, 0, 1, 2), None, stride, padding)
+    if subm:
+        mask = H.dense_from_rows(np.ones((idx.shape[0], 1)), idx, B, shape)
+        ref = ref * mask
+    tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=2e-3)
+    torch.testing.assert_close(dense_y.detach().double().cpu(), ref.detach(), **tol)
+    up = torch.randn(ref.shape, dtype=torch.float64, generator=torch.Generator().manual_seed(0))
+    if subm:
+        up = up * mask
+    else:
+        up = up * (ref.detach().abs().sum(1, keepdim=True) != 0)      # grads only at active outputs
+    (ref * up).sum().backward()
+    (dense_y * up.to(G.DEV).to(dtype)).sum().backward()
+    gtol = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(f.grad.double().cpu(), f64.grad, **gtol)
+    torch.testing.assert_close(conv.weight.grad.double().cpu(), w64.grad, **gtol)
+
+
+def test_sequential_rule_reuse_and_plain_modules():
+    B, shape = 2, [8, 16, 12]
+    idx, feat = _inputs(2, B, shape, 4)
+    net = sphconv.SparseSequential(
+        sphconv.SubMConv3d(4, 8, 3, indice_key="s1"),
+        torch.nn.BatchNorm1d(8), torch.nn.ReLU(),
+        sphconv.SubMConv3d(8, 8, 3, indice_key="s1"),
+        torch.nn.BatchNorm1d(8), torch.nn.ReLU(),
+        sphconv.SparseConv3d(8, 16, 3, stride=2, padding=1),
+    ).to(G.DEV).eval()
+    x = sphconv.SparseConvTensor(G.t(feat), shape, B, indices=G.t(idx))
+    with torch.no_grad():
+        y = net(x)
+    assert "s1" in x.rule_cache and net[0].rule_book is net[3].rule_book
+    assert [y.D, y.W, y.H] == [4, 8, 6] and y.feature.shape[1] == 16
+    # dense re-computation
+    with torch.no_grad():
+        d = x.dense().cpu().double()
+        mask = (H.dense_from_rows(np.ones((idx.shape[0], 1)), idx, B, shape) != 0).double()
+        for i in (0, 3):
+            w = net[i].weight.detach().cpu().double().permute(4, 3, 0, 1, 2)
+            d = torch.nn.functional.conv3d(d, w, None, 1, 1) * mask
+            bn = net[i + 1]
+            s = (bn.weight / torch.sqrt(bn.running_var + bn.eps)).cpu().double()
+            sh = (bn.bias - bn.running_mean * bn.weight / torch.sqrt(bn.running_var + bn.eps)).cpu().double()
+            d = torch.relu(d * s[None, :, None, None, None] + sh[None, :, None, None, None]) * mask
+        w = net[6].weight.detach().cpu().double().permute(4, 3, 0, 1, 2)
+        d = torch.nn.functional.conv3d(d, w, None, 2, 1)
+    torch.testing.assert_close(y.dense().cpu().double(), d, rtol=1e-4, atol=1e-5)
+    assert net[0].rule_size.shape == (4 * 8, 27)
+
+
+def test_rangevoxel_bridge():
+    B, H_, W_, D_, C = 2, 6, 9, 11, 3
+    idx, feat = _inputs(3, B, [H_, W_, D_], C, p=0.3)
+    x = sphconv.SparseConvTensor(G.t(feat), [H_, W_, D_], B, indices=G.t(idx))
+    rv = sphconv.RangeVoxel.from_sparse(x)
+    assert tuple(rv.shape) == (B, C, D_, H_, W_)
+    back = rv.to_sparse()
+    assert torch.equal(back.z_idx, x.z_idx) and torch.equal(back.z_ptr, x.z_ptr)
+    assert torch.equal(back.feature, x.feature)
+    assert torch.equal(rv.dense(), x.dense().permute(0, 1, 4, 2, 3))
+    with pytest.raises(AssertionError):
+        sphconv.RangeVoxel(rv.feature, rv.depth, rv.thick, (B, C + 1, D_, H_, W_))
