@@ -55,9 +55,11 @@ __device__ __forceinline__ typename Traits<DT>::acc4 mfma_step(int4v a, int4v b,
 template <>
 __device__ __forceinline__ float4v mfma_step<SPH_F32>(int4v a, int4v b, float4v d)
 {
-#pragma unroll
-    for (int j = 0; j < 4; j++)
-        d = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[j]), __builtin_bit_cast(float, b[j]), d, 0, 0, 0);
+    const float4v af = __builtin_bit_cast(float4v, a), bf = __builtin_bit_cast(float4v, b);
+    d = __builtin_amdgcn_mfma_f32_16x16x4f32(af.x, bf.x, d, 0, 0, 0);
+    d = __builtin_amdgcn_mfma_f32_16x16x4f32(af.y, bf.y, d, 0, 0, 0);
+    d = __builtin_amdgcn_mfma_f32_16x16x4f32(af.z, bf.z, d, 0, 0, 0);
+    d = __builtin_amdgcn_mfma_f32_16x16x4f32(af.w, bf.w, d, 0, 0, 0);
     return d;
 }
 template <>

@@ -169,7 +169,19 @@ def test_fp32_backward(ic, oc, subm, kernel, stride, padding):
     # reference entry point: weight pre-permuted to [KV,oC,iC]
     d_feat, d_w = ext.rule_conv_backward(G.t(g), G.t(feat), G.t(w_perm), book, None, tgs)
     np.testing.assert_allclose(d_feat.cpu().numpy(), d_feat_o, rtol=1e-5, atol=1e-5)
-    np.testing.assert_allclose(d_w.cpu().numpy(), d_w_o, rtol=1e-4, atol=1e-4)
+    # d_weight sums thousands of products that cancel: both fp32 evaluations (oracle and
+    # GPU, different association) are held to 1e-5 of the sum of absolute products,
+    # measured against the float64 definition
+    tri = G.oracle_triples(rules, rule_size)
+    dw64 = np.zeros((kv, ic, oc))
+    mag = np.zeros((kv, ic, oc))
+    f64, g64 = feat.astype(np.float64), g.astype(np.float64)
+    for k in np.unique(tri[:, 0]):
+        s = tri[tri[:, 0] == k]
+        dw64[k] = f64[s[:, 1]].T @ g64[s[:, 2]]
+        mag[k] = np.abs(f64[s[:, 1]]).T @ np.abs(g64[s[:, 2]])
+    assert (np.abs(d_w.cpu().numpy() - dw64) <= 1e-5 * mag + 1e-6).all()
+    assert (np.abs(d_w_o - dw64) <= 1e-5 * mag + 1e-6).all()
     # same through padded rules
     pr, ps = book.padded((2, 2))
     d_feat2, d_w2 = ext.rule_conv_backward(G.t(g), G.t(feat), G.t(w_perm), pr, ps, tgs)
