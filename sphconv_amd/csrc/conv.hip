@@ -169,13 +169,39 @@ __device__ __forceinline__ typename Traits<DT>::elem to_elem(float v)
     return (elem)v;
 }
 
-template <sph_dtype DT, int NW>
+// Adds the four accumulators a lane holds after a transposed MFMA (four consecutive
+// output columns of ONE owner row) into the LDS tile with a single 16-byte
+// read-modify-write.  The address range belongs to this wave only, so additions
+// happen in program order and the sum is reproducible.  (LDS float atomics
+// serialise per lane and measured 2x slower.)
+template <sph_dtype DT>
+__device__ __forceinline__ void acc_add4(uint32_t *p, typename Traits<DT>::acc4 d)
+{
+    typedef typename Traits<DT>::acc4 acc4;
+    acc4 v = *(acc4 *)p;
+    v += d;
+    *(acc4 *)p = v;
+}
+
+constexpr int kMetaGroups = 32; // groups whose indices are staged in LDS at a time
+constexpr int kUnroll = 4;      // groups whose fragments are in flight together
+
+// The MFMA is issued transposed: D^T[16 owner columns, 16 pairs] = W^T x A^T, so
+// lane l ends up with columns 4*(l/16)..+3 of pair l%16.
+//
+// NSTEP > 0: number of 64-byte steps per gathered row, known at compile time (the
+// fragments of kUnroll groups are then loaded before the first MFMA);
+// NSTEP == 0: any row length, one group at a time.
+template <sph_dtype DT, int NW, int NSTEP>
 __global__ __launch_bounds__(NW * kWave) void conv_apply_kernel(ConvArgs a)
 {
     typedef typename Traits<DT>::elem elem;
     typedef typename Traits<DT>::acc4 acc4;
-    constexpr int LDW = NW * 16 + 4; // accumulator row stride in 32-bit words
-    extern __shared__ uint32_t s_acc[]; // [R][LDW]
+    constexpr int LDW = NW * 16 + 4; // accumulator row stride in 32-bit words (16-byte multiple)
+    extern __shared__ __attribute__((aligned(16))) uint32_t s_acc[]; // [R][LDW]
+    __shared__ int s_k[kMetaGroups];
+    __shared__ int2 s_meta[kMetaGroups * SPH_GROUP]; // (gathered row, owner row - r0)
+    __shared__ int4v s_afrag[kUnroll * (NSTEP > 0 ? NSTEP : 1) * kWave]; // gathered fragments of one chunk
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -185,32 +211,99 @@ __global__ __launch_bounds__(NW * kWave) void conv_apply_kernel(ConvArgs a)
     const int nrows = min(R, a.book.rows - r0);
 
     // each wave clears and later updates only its own 16 columns
-    for (int i = lane; i < R * 16; i += kWave) s_acc[(i >> 4) * LDW + wave * 16 + (i & 15)] = 0u;
+    for (int i = lane; i < R * 4; i += kWave)
+        *(int4v *)&s_acc[(i >> 2) * LDW + wave * 16 + (i & 3) * 4] = int4v{0, 0, 0, 0};
 
     const int ngrp = a.book.tile_ngrp[tile];
     const long gb0 = (long)tile * a.cap;
-    const int col = wave * 16 + (lane & 15);
-    for (int g = 0; g < ngrp; g++) {
-        const int k = a.book.grp_k[gb0 + g];
-        const long slot = (gb0 + g) * SPH_GROUP;
-        const int in_row = a.book.grp_gather[slot + (lane & 15)];
-        const int4v own = *(const int4v *)(a.book.grp_owner + slot + (lane >> 4) * 4);
-        acc4 d = {0, 0, 0, 0};
-        const char *wk = a.wp + ((long)k * a.nsteps * NW + wave) * (kWave * 16) + lane * 16;
-        for (int st = 0; st < a.nsteps; st++) {
-            int4v fa = load_a_frag<DT>(a, in_row, st, lane);
-            int4v fb = *(const int4v *)(wk + (long)st * NW * (kWave * 16));
-            d = mfma_step<DT>(fa, fb, d);
+    const int acc_col = wave * 16 + (lane >> 4) * 4;
+    const char *wlane = a.wp + (long)wave * (kWave * 16) + lane * 16;
+    const long wstep = (long)NW * (kWave * 16);           // bytes between steps of one offset
+    const int nsteps = NSTEP > 0 ? NSTEP : a.nsteps;
+
+    for (int c0 = 0; c0 < ngrp; c0 += kMetaGroups) {
+        const int nc = min(kMetaGroups, ngrp - c0);
+        if (c0) __syncthreads(); // every wave is done with the previous chunk's indices
+        for (int i = tid; i < nc * SPH_GROUP; i += NW * kWave) {
+            int gi = a.book.grp_gather[(gb0 + c0) * SPH_GROUP + i];
+            int rl = a.book.grp_owner[(gb0 + c0) * SPH_GROUP + i] - r0;
+            if ((unsigned)rl >= (unsigned)nrows || (unsigned)gi >= (unsigned)a.feat_rows) gi = rl = -1;
+            s_meta[i] = make_int2(gi, rl);
         }
+        for (int i = tid; i < nc; i += NW * kWave) s_k[i] = a.book.grp_k[gb0 + c0 + i];
+        __syncthreads();
+
+        if (NSTEP > 0) {
+            // Groups are taken kUnroll at a time.  Each group's 16 rows are gathered by ONE
+            // wave (16 B per lane, already in MFMA operand order) and handed to the other
+            // waves through LDS, so a row crosses the vector memory path once per workgroup
+            // instead of once per wave.  Gathers and weight fragments of the next chunk are
+            // in flight while the current chunk is multiplied.
+            constexpr int NS = NSTEP > 0 ? NSTEP : 1;
+            constexpr int MAXG = (kUnroll + NW - 1) / NW; // groups of a chunk gathered by one wave
+            int4v a_next[MAXG][NS], w_next[kUnroll][NS], w_cur[kUnroll][NS];
+            auto gather_chunk = [&](int g0) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            int rl = own[r] - r0;
-            if ((unsigned)rl < (unsigned)nrows) {
-                uint32_t *p = &s_acc[rl * LDW + col];
-                if (DT == SPH_I8)
-                    *p = (uint32_t)((int32_t)*p + (int32_t)d[r]);
-                else
-                    *p = __builtin_bit_cast(uint32_t, __builtin_bit_cast(float, *p) + (float)d[r]);
+                for (int j = 0; j < MAXG; j++) {
+                    const int u = wave + j * NW;
+                    const int in_row = (u < kUnroll && g0 + u < nc) ? s_meta[(g0 + u) * SPH_GROUP + (lane & 15)].x : -1;
+#pragma unroll
+                    for (int st = 0; st < NS; st++) a_next[j][st] = load_a_frag<DT>(a, in_row, st, lane);
+                }
+            };
+            auto weights_chunk = [&](int g0) {
+#pragma unroll
+                for (int u = 0; u < kUnroll; u++) {
+                    const int k = (g0 + u < nc) ? s_k[g0 + u] : 0;
+                    const char *wk = wlane + (long)k * NS * wstep;
+#pragma unroll
+                    for (int st = 0; st < NS; st++) w_next[u][st] = *(const int4v *)(wk + st * wstep);
+                }
+            };
+            gather_chunk(0);
+            weights_chunk(0);
+            for (int g = 0; g < nc; g += kUnroll) {
+#pragma unroll
+                for (int j = 0; j < MAXG; j++) {
+                    const int u = wave + j * NW;
+                    if (u < kUnroll) {
+#pragma unroll
+                        for (int st = 0; st < NS; st++) s_afrag[(u * NS + st) * kWave + lane] = a_next[j][st];
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < kUnroll; u++)
+#pragma unroll
+                    for (int st = 0; st < NS; st++) w_cur[u][st] = w_next[u][st];
+                __syncthreads();
+                if (g + kUnroll < nc) {
+                    gather_chunk(g + kUnroll);
+                    weights_chunk(g + kUnroll);
+                }
+#pragma unroll
+                for (int u = 0; u < kUnroll; u++) {
+                    if (g + u < nc) {
+                        acc4 d = {0, 0, 0, 0};
+#pragma unroll
+                        for (int st = 0; st < NS; st++)
+                            d = mfma_step<DT>(w_cur[u][st], s_afrag[(u * NS + st) * kWave + lane], d);
+                        const int rl = s_meta[(g + u) * SPH_GROUP + (lane & 15)].y;
+                        if (rl >= 0) acc_add4<DT>(&s_acc[rl * LDW + acc_col], d);
+                    }
+                }
+                __syncthreads(); // the fragments are consumed before the next chunk overwrites them
+            }
+        } else {
+            for (int g = 0; g < nc; g++) {
+                const int2 m = s_meta[g * SPH_GROUP + (lane & 15)];
+                const char *wk = wlane + (long)s_k[g] * nsteps * wstep;
+                acc4 d = {0, 0, 0, 0};
+                for (int st = 0; st < nsteps; st++) {
+                    int4v fa = load_a_frag<DT>(a, m.x, st, lane);
+                    int4v fb = *(const int4v *)(wk + st * wstep);
+                    d = mfma_step<DT>(fb, fa, d);
+                }
+                if (m.y >= 0) acc_add4<DT>(&s_acc[m.y * LDW + acc_col], d);
             }
         }
     }
@@ -375,14 +468,28 @@ inline int set_lds(K kernel, size_t bytes)
     return SPH_OK;
 }
 
+template <sph_dtype DT, int NW, int NSTEP>
+int launch_conv_ns(const ConvArgs &a, int ntiles, hipStream_t st)
+{
+    size_t lds = (size_t)R * (NW * 16 + 4) * sizeof(uint32_t);
+    int rc = set_lds(conv_apply_kernel<DT, NW, NSTEP>, lds);
+    if (rc) return rc;
+    hipLaunchKernelGGL((conv_apply_kernel<DT, NW, NSTEP>), dim3(ntiles), dim3(NW * kWave), lds, st, a);
+    return sph_check_launch("sph_conv_apply");
+}
+
 template <sph_dtype DT, int NW>
 int launch_conv(const ConvArgs &a, int ntiles, hipStream_t st)
 {
-    size_t lds = (size_t)R * (NW * 16 + 4) * sizeof(uint32_t);
-    int rc = set_lds(conv_apply_kernel<DT, NW>, lds);
-    if (rc) return rc;
-    hipLaunchKernelGGL((conv_apply_kernel<DT, NW>), dim3(ntiles), dim3(NW * kWave), lds, st, a);
-    return sph_check_launch("sph_conv_apply");
+    if (a.aligned_in) {
+        switch (a.nsteps) {
+        case 1: return launch_conv_ns<DT, NW, 1>(a, ntiles, st);
+        case 2: return launch_conv_ns<DT, NW, 2>(a, ntiles, st);
+        case 4: return launch_conv_ns<DT, NW, 4>(a, ntiles, st);
+        default: break;
+        }
+    }
+    return launch_conv_ns<DT, NW, 0>(a, ntiles, st);
 }
 
 template <sph_dtype DT>
