@@ -33,22 +33,29 @@ __device__ __forceinline__ void fiber_range(const int32_t *ptr, int c, int rows,
     if (start > end) start = end;
 }
 
-// First column c in [0, n) with a[c] > target (n if none), found by all
-// kThreads threads of the block together: every round probes kThreads evenly
-// spaced positions of the remaining window, so 2-3 rounds cover any grid.
-// s_tmp: one LDS int.  Must be called by the whole block.
-__device__ int block_upper_bound(const int32_t *a, int n, int target, int *s_tmp)
+// Narrows down the first column c in [0, n) with a[c] > target (n if none): returns
+// lo <= c with c - lo < max_span.  All kThreads threads of the block work together:
+// every round probes kThreads evenly spaced positions of the remaining window, so a
+// round cuts the window by a factor of kThreads.  (Probes are scattered, one cache
+// line each, and cost far more in the vector memory path than the coalesced column
+// walk that follows; hence few probes and an early stop.)  max_span = 1 gives the
+// exact column.  s_tmp: one LDS int.  Must be called by the whole block.
+__device__ int block_upper_bound(const int32_t *a, int n, int target, int max_span, int *s_tmp)
 {
     int lo = 0, hi = n;
     const int tid = threadIdx.x;
-    while (hi > lo) {
+    while (hi - lo >= max_span) {
         int span = hi - lo;
         int step = (span + kThreads - 1) / kThreads;
         long pos = (long)lo + (long)tid * step;
-        bool pred = (pos < hi) ? (a[pos] > target) : true;
+        int val = (pos < hi) ? a[pos] : 0x7fffffff; // positions >= hi are known to exceed
+        int first = (val > target) ? tid : kThreads;
         if (tid == 0) *s_tmp = kThreads;
         __syncthreads();
-        if (pred) atomicMin(s_tmp, tid);
+        // one LDS atomic per wave: reduce to the wave's smallest index first
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) first = min(first, __shfl_xor(first, off, kWave));
+        if ((tid & (kWave - 1)) == 0 && first < kThreads) atomicMin(s_tmp, first);
         __syncthreads();
         int f = *s_tmp;
         __syncthreads();
@@ -70,63 +77,102 @@ __device__ int block_upper_bound(const int32_t *a, int n, int target, int *s_tmp
 // nbr[row_local * KV + k] = gathered row or -1 for the `nrows` rows of tile
 // `tile` (first row r0).  Emits the tile's groups: per k, rows in ascending
 // order, 16 per group, last group padded with -1.
-// LDS scratch: s_cnt[KV], s_goff[KV + 1].
+//   pass 1: per k a 128-bit occupancy mask of the rows (wave ballots) and its count;
+//   scan  : first group of every k;
+//   pass 2: one thread per output SLOT finds its k and its rank in the k-list,
+//           selects the rank-th set bit of the mask and stores -- consecutive
+//           threads store consecutive slots, so the book is written coalesced.
 // ---------------------------------------------------------------------------
-__device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int tile, int cap,
-                            int *s_cnt, int *s_goff, const sph_book &book)
+struct EmitScratch {
+    unsigned long long mask[SPH_MAX_KV][R / 64];
+    int cnt[SPH_MAX_KV];
+    int goff[SPH_MAX_KV + 1];
+    unsigned char gk[SPH_MAX_KV * (R / SPH_GROUP)];
+};
+
+// Position of the j-th (0-based) set bit of m; m must have more than j bits set.
+__device__ __forceinline__ int select_bit(unsigned long long m, int j)
 {
+    int base = 0;
+#pragma unroll
+    for (int w = 32; w >= 1; w >>= 1) {
+        unsigned long long low = m & ((1ull << w) - 1ull);
+        int c = __popcll(low);
+        if (j >= c) {
+            j -= c;
+            m >>= w;
+            base += w;
+        } else {
+            m = low;
+        }
+    }
+    return base;
+}
+
+__device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int tile, int cap,
+                            EmitScratch &sc, const sph_book &book)
+{
+    static_assert(R == 128, "the occupancy masks assume 128 rows per tile");
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
 
     for (int k = wave; k < KV; k += kWaves) {
-        int cnt = 0;
-        for (int h = 0; h < R; h += kWave) {
-            int row = h + lane;
-            int v = (row < nrows) ? nbr[row * KV + k] : -1;
-            cnt += __popcll(__ballot(v >= 0));
+        int r_lo = lane, r_hi = kWave + lane;
+        unsigned long long m0 = __ballot(r_lo < nrows && nbr[r_lo * KV + k] >= 0);
+        unsigned long long m1 = __ballot(r_hi < nrows && nbr[r_hi * KV + k] >= 0);
+        if (lane == 0) {
+            sc.mask[k][0] = m0;
+            sc.mask[k][1] = m1;
+            sc.cnt[k] = __popcll(m0) + __popcll(m1);
         }
-        if (lane == 0) s_cnt[k] = cnt;
     }
     __syncthreads();
-    if (tid == 0) {
-        int g = 0;
-        for (int k = 0; k < KV; k++) {
-            s_goff[k] = g;
-            g += (s_cnt[k] + SPH_GROUP - 1) / SPH_GROUP;
+    if (wave == 0) {
+        // exclusive scan of the per-offset group counts by one wave (KV <= 128: two passes)
+        int carry = 0;
+        for (int k0 = 0; k0 < KV; k0 += kWave) {
+            int k = k0 + lane;
+            int v = (k < KV) ? (sc.cnt[k] + SPH_GROUP - 1) / SPH_GROUP : 0;
+            int incl = v;
+#pragma unroll
+            for (int off = 1; off < kWave; off <<= 1) {
+                int t = __shfl_up(incl, off, kWave);
+                if (lane >= off) incl += t;
+            }
+            if (k < KV) {
+                sc.goff[k] = carry + incl - v;
+                for (int g = 0; g < v; g++) sc.gk[carry + incl - v + g] = (unsigned char)k;
+            }
+            carry += __shfl(incl, kWave - 1, kWave);
         }
-        s_goff[KV] = g;
-        book.tile_ngrp[tile] = g;
+        if (lane == 0) {
+            sc.goff[KV] = carry;
+            book.tile_ngrp[tile] = carry;
+        }
     }
     __syncthreads();
 
+    const int ngrp = sc.goff[KV];
     const long gbase_tile = (long)tile * cap;
-    for (int k = wave; k < KV; k += kWaves) {
-        const int cnt = s_cnt[k];
-        if (cnt == 0) continue;
-        const long slot0 = (gbase_tile + s_goff[k]) * SPH_GROUP;
-        int pos = 0;
-        for (int h = 0; h < R; h += kWave) {
-            int row = h + lane;
-            int v = (row < nrows) ? nbr[row * KV + k] : -1;
-            unsigned long long m = __ballot(v >= 0);
-            if (v >= 0) {
-                int my = pos + __popcll(m & ((1ull << lane) - 1ull));
-                book.grp_gather[slot0 + my] = v;
-                book.grp_owner[slot0 + my] = r0 + row;
-            }
-            pos += __popcll(m);
+    for (int slot = tid; slot < ngrp * SPH_GROUP; slot += kThreads) {
+        const int g = slot / SPH_GROUP;
+        const int k = sc.gk[g];
+        const int j = (g - sc.goff[k]) * SPH_GROUP + (slot & (SPH_GROUP - 1));
+        int gat = -1, own = -1;
+        if (j < sc.cnt[k]) {
+            const unsigned long long m0 = sc.mask[k][0];
+            const int c0 = __popcll(m0);
+            const int row = j < c0 ? select_bit(m0, j) : 64 + select_bit(sc.mask[k][1], j - c0);
+            gat = nbr[row * KV + k];
+            own = r0 + row;
         }
-        int padded = (cnt + SPH_GROUP - 1) / SPH_GROUP * SPH_GROUP;
-        if (lane < padded - cnt) {
-            book.grp_gather[slot0 + cnt + lane] = -1;
-            book.grp_owner[slot0 + cnt + lane] = -1;
-        }
-        int ng = padded / SPH_GROUP;
-        for (int g = lane; g < ng; g += kWave) book.grp_k[gbase_tile + s_goff[k] + g] = k;
+        book.grp_gather[gbase_tile * SPH_GROUP + slot] = gat;
+        book.grp_owner[gbase_tile * SPH_GROUP + slot] = own;
     }
+    for (int g = tid; g < ngrp; g += kThreads) book.grp_k[gbase_tile + g] = sc.gk[g];
     for (int k = tid; k <= KV; k += kThreads)
-        book.tile_koff[(long)tile * (KV + 1) + k] = (uint16_t)s_goff[k];
+        book.tile_koff[(long)tile * (KV + 1) + k] = (uint16_t)sc.goff[k];
 }
 
 // ---------------------------------------------------------------------------
@@ -150,13 +196,15 @@ struct BuildArgs {
     sph_book book;
 };
 
+constexpr int kJoinItems = 5; // (row, k0, k1) items a thread joins per pass, all loads of a pass in flight together
+
 template <bool TRANSPOSED>
 __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
 {
     extern __shared__ int32_t s_nbr[]; // [R * KV]
     __shared__ int s_col[R];
     __shared__ int s_b[R], s_c0[R], s_c1[R], s_z[R];
-    __shared__ int s_cnt[SPH_MAX_KV], s_goff[SPH_MAX_KV + 1];
+    __shared__ EmitScratch s_emit;
     __shared__ int s_tmp, s_flag;
 
     const int tid = threadIdx.x;
@@ -168,75 +216,115 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     const int nrows = r1 - r0;
     const int q_ncol = a.B * a.Q.n0 * a.Q.n1;
 
+    // the tile's own S2 coordinates do not depend on the column search: fetch them first
+    const int my_z = (tid < nrows) ? a.q_idx[r0 + tid] : 0;
+
     for (int i = tid; i < R * KV; i += kThreads) s_nbr[i] = -1;
     for (int i = tid; i < R; i += kThreads) s_col[i] = -1;
+    __syncthreads();
 
-    // 1. rows -> columns
-    int c_first = block_upper_bound(a.q_ptr, q_ncol, r0, &s_tmp);
+    // 1. rows -> columns.  The walk below tolerates starting early (columns before the
+    // tile hold none of its rows), so the search stops once the window is below one
+    // walk step: a single round of probes for grids of up to 131072 columns.
+    constexpr int kWalk = 2 * kThreads; // columns per walk step, two consecutive ones per thread
+    int c_first = block_upper_bound(a.q_ptr, q_ncol, r0, kWalk, &s_tmp);
     bool done = (c_first >= q_ncol);
-    for (int cb = c_first; !done; cb += kThreads) {
-        int c = cb + tid;
-        int last = min(cb + kThreads - 1, q_ncol - 1);
+    for (int cb = c_first; !done; cb += kWalk) {
+        const int last = min(cb + kWalk - 1, q_ncol - 1);
+        const int c = cb + 2 * tid;
         if (c <= last) {
-            int s, e;
-            fiber_range(a.q_ptr, c, a.q_rows, s, e);
-            int lo = max(s, r0), hi = min(e, r1);
-            for (int r = lo; r < hi; r++) s_col[r - r0] = c;
-            if (c == last) s_flag = (e >= r1) || (last == q_ncol - 1);
+            // q_ptr[c-1], q_ptr[c], q_ptr[c+1] bound the fibers of columns c and c+1
+            int p0 = c ? clampi(a.q_ptr[c - 1], 0, a.q_rows) : 0;
+            int p1 = clampi(a.q_ptr[c], 0, a.q_rows);
+            int p2 = (c + 1 <= last) ? clampi(a.q_ptr[c + 1], 0, a.q_rows) : p1;
+            if (p1 < p0) p1 = p0;
+            if (p2 < p1) p2 = p1;
+            for (int r = max(p0, r0); r < min(p1, r1); r++) s_col[r - r0] = c;
+            for (int r = max(p1, r0); r < min(p2, r1); r++) s_col[r - r0] = c + 1;
+            if (c == last || c + 1 == last) s_flag = (p2 >= r1) || (last == q_ncol - 1);
         }
         __syncthreads();
         done = s_flag != 0;
         __syncthreads();
     }
-    __syncthreads();
-    for (int i = tid; i < nrows; i += kThreads) {
-        int c = s_col[i];
+    if (tid < nrows) {
+        int c = s_col[tid];
         if (c >= 0) {
             int b = c / (a.Q.n0 * a.Q.n1);
             int rem = c - b * (a.Q.n0 * a.Q.n1);
-            s_b[i] = b;
-            s_c0[i] = rem / a.Q.n1;
-            s_c1[i] = rem % a.Q.n1;
-            s_z[i] = a.q_idx[r0 + i];
+            s_b[tid] = b;
+            s_c0[tid] = rem / a.Q.n1;
+            s_c1[tid] = rem % a.Q.n1;
+            s_z[tid] = my_z;
         }
     }
     __syncthreads();
 
-    // 2. join: item = (k01, row); consecutive lanes take consecutive rows
-    for (int it = tid; it < K01 * R; it += kThreads) {
-        int rl = it & (R - 1);
-        int k01 = it / R;
-        if (rl >= nrows || s_col[rl] < 0) continue;
-        int k0 = k01 / a.cv.K1, k1 = k01 - k0 * a.cv.K1;
-        int y0, y1;
-        if (!TRANSPOSED) {
-            y0 = s_c0[rl] * a.cv.s0 - a.cv.p0 + k0;
-            y1 = s_c1[rl] * a.cv.s1 - a.cv.p1 + k1;
-        } else {
-            int t0 = s_c0[rl] + a.cv.p0 - k0, t1 = s_c1[rl] + a.cv.p1 - k1;
-            if (t0 < 0 || t1 < 0 || t0 % a.cv.s0 || t1 % a.cv.s1) continue;
-            y0 = t0 / a.cv.s0;
-            y1 = t1 / a.cv.s1;
+    // 2. join.  item = (k01, row), consecutive lanes take consecutive rows.  Per pass a
+    // thread first issues the two fiber-bound loads of all its items, then the first
+    // three S2 coordinates of every fiber, and only then compares; longer fibers finish
+    // in a loop.
+    for (int base = 0; base < K01 * R; base += kThreads * kJoinItems) {
+        int ps[kJoinItems], len[kJoinItems], slot[kJoinItems], zz[kJoinItems];
+        int raw_e[kJoinItems], raw_s[kJoinItems];
+        bool ok[kJoinItems];
+#pragma unroll
+        for (int j = 0; j < kJoinItems; j++) {
+            const int it = base + j * kThreads + tid;
+            const int rl = it & (R - 1);
+            const int k01 = it / R;
+            ok[j] = it < K01 * R && rl < nrows && s_col[rl] >= 0;
+            const int rr = ok[j] ? rl : 0;
+            const int k0 = k01 / a.cv.K1, k1 = k01 - k0 * a.cv.K1;
+            int y0, y1;
+            if (!TRANSPOSED) {
+                y0 = s_c0[rr] * a.cv.s0 - a.cv.p0 + k0;
+                y1 = s_c1[rr] * a.cv.s1 - a.cv.p1 + k1;
+            } else {
+                int t0 = s_c0[rr] + a.cv.p0 - k0, t1 = s_c1[rr] + a.cv.p1 - k1;
+                if (t0 < 0 || t1 < 0 || t0 % a.cv.s0 || t1 % a.cv.s1) ok[j] = false;
+                y0 = t0 / a.cv.s0;
+                y1 = t1 / a.cv.s1;
+            }
+            if (y0 < 0 || y0 >= a.P.n0 || y1 < 0 || y1 >= a.P.n1) ok[j] = false;
+            const int pc = ok[j] ? (s_b[rr] * a.P.n0 + y0) * a.P.n1 + y1 : 0;
+            raw_e[j] = a.p_ptr[pc];
+            raw_s[j] = pc ? a.p_ptr[pc - 1] : 0;
+            slot[j] = rr * KV + k01 * a.cv.K2;
+            zz[j] = s_z[rr];
         }
-        if (y0 < 0 || y0 >= a.P.n0 || y1 < 0 || y1 >= a.P.n1) continue;
-        int pc = (s_b[rl] * a.P.n0 + y0) * a.P.n1 + y1;
-        int ps, pe;
-        fiber_range(a.p_ptr, pc, a.p_rows, ps, pe);
-        const int z = s_z[rl];
-        for (int e = ps; e < pe; e++) {
-            int zz = a.p_idx[e];
-            int k2;
-            if (!TRANSPOSED)
-                k2 = zz - (z * a.cv.s2 - a.cv.p2); // zz is the input S2 coordinate
-            else
-                k2 = z + a.cv.p2 - zz * a.cv.s2;   // zz is the output S2 coordinate
-            if (k2 >= 0 && k2 < a.cv.K2) s_nbr[rl * KV + k01 * a.cv.K2 + k2] = e;
+        int z0[kJoinItems], z1[kJoinItems], z2[kJoinItems];
+#pragma unroll
+        for (int j = 0; j < kJoinItems; j++) {
+            int e = clampi(raw_e[j], 0, a.p_rows), st = clampi(raw_s[j], 0, a.p_rows);
+            if (st > e) st = e;
+            ps[j] = st;
+            len[j] = ok[j] ? e - st : 0;
+            z0[j] = z1[j] = z2[j] = 0;
+            if (len[j] > 0) z0[j] = a.p_idx[st];
+            if (len[j] > 1) z1[j] = a.p_idx[st + 1];
+            if (len[j] > 2) z2[j] = a.p_idx[st + 2];
+        }
+#pragma unroll
+        for (int j = 0; j < kJoinItems; j++) {
+            // k2 of a gathered-side entry with S2 coordinate v: forward v is an input
+            // coordinate (k2 = v - (z*s2 - p2)), transposed v is an output coordinate
+            // (k2 = z + p2 - v*s2)
+            const int off = TRANSPOSED ? zz[j] + a.cv.p2 : -(zz[j] * a.cv.s2 - a.cv.p2);
+            const int mul = TRANSPOSED ? -a.cv.s2 : 1;
+            if (len[j] > 0) { int k2 = off + mul * z0[j]; if (k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j]; }
+            if (len[j] > 1) { int k2 = off + mul * z1[j]; if (k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j] + 1; }
+            if (len[j] > 2) { int k2 = off + mul * z2[j]; if (k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j] + 2; }
+            for (int e = 3; e < len[j]; e++) {
+                int k2 = off + mul * a.p_idx[ps[j] + e];
+                if (k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j] + e;
+            }
         }
     }
     __syncthreads();
 
     // 3. compaction
-    emit_groups(s_nbr, nrows, r0, KV, tile, a.cap, s_cnt, s_goff, a.book);
+    emit_groups(s_nbr, nrows, r0, KV, tile, a.cap, s_emit, a.book);
 }
 
 // Book builder from a global neighbour table nbr[rows, KV] (used when the rules
@@ -245,13 +333,13 @@ __global__ __launch_bounds__(kThreads) void book_from_nbr_kernel(const int32_t *
                                                                  int cap, sph_book book)
 {
     extern __shared__ int32_t s_nbr[];
-    __shared__ int s_cnt[SPH_MAX_KV], s_goff[SPH_MAX_KV + 1];
+    __shared__ EmitScratch s_emit;
     const int tile = blockIdx.x;
     const int r0 = tile * R;
     const int nrows = min(R, rows - r0);
     for (int i = threadIdx.x; i < nrows * KV; i += kThreads) s_nbr[i] = nbr[(long)r0 * KV + i];
     __syncthreads();
-    emit_groups(s_nbr, nrows, r0, KV, tile, cap, s_cnt, s_goff, book);
+    emit_groups(s_nbr, nrows, r0, KV, tile, cap, s_emit, book);
 }
 
 // ---------------------------------------------------------------------------
