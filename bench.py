@@ -21,6 +21,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the two candidates for "dominant kernel" at the default workload
+# (seed 0), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script scaled by a
+# 256 MiB copy (factors 2.000 / 1.000); commands and raw values: profiles/bench_headline_subm64_f16.md.
+# None for any other workload.
+MEASURED_TRAFFIC_BYTES = {"conv": 13459 * 1024 * 2 + 11924 * 1024, "rules": 2221 * 1024 * 2 + 3351 * 1024}
 
 
 def parse():
@@ -31,6 +36,9 @@ def parse():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three 256 MiB device-to-device copies (a kernel of known HBM traffic, "
+                         "to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     return ap.parse_args()
 
 
@@ -114,6 +122,14 @@ def main():
     w = torch.tensor(rng.standard_normal((27, ic, oc)) * np.sqrt(2.0 / (27 * ic)), dtype=torch.float32,
                      device=dev).half()
 
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     def step():
         book = RuleBook.build_subm(z_idx, z_ptr, B, shape, [3, 3, 3])
         return book, ext.rule_conv(feat, w, book, None, n)
@@ -155,12 +171,13 @@ def main():
     rule_bytes = 4 * z_ptr.numel() + 4 * n + 8 * P + nt * (4 + 2 * 28)
     conv_flops = 2.0 * P * ic * oc
     if conv_ms >= rulegen_ms:
-        dom = {"kernel": "conv_apply_kernel<f16,4>", "bytes": conv_bytes, "ms": conv_ms}
+        dom = {"kernel": "conv_apply_kernel<f16,4,2>", "bytes": conv_bytes, "ms": conv_ms, "key": "conv"}
     else:
-        dom = {"kernel": "build_book_kernel<false>", "bytes": rule_bytes, "ms": rulegen_ms}
+        dom = {"kernel": "build_book_kernel<false>", "bytes": rule_bytes, "ms": rulegen_ms, "key": "rules"}
     achieved = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
     roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": dom["kernel"],
+                "frac": achieved / HBM_PEAK_GBS,
+                "traffic": MEASURED_TRAFFIC_BYTES[dom["key"]] if args.seed == 0 else None, "kernel": dom["kernel"],
                 "algorithmic_bytes": dom["bytes"], "kernel_ms": dom["ms"]}
 
     result = {
