@@ -171,7 +171,7 @@ def main():
     rule_bytes = 4 * z_ptr.numel() + 4 * n + 8 * P + nt * (4 + 2 * 28)
     conv_flops = 2.0 * P * ic * oc
     if conv_ms >= rulegen_ms:
-        dom = {"kernel": "conv_apply_kernel<f16,4,2>", "bytes": conv_bytes, "ms": conv_ms, "key": "conv"}
+        dom = {"kernel": "conv_wave_kernel<f16,2,4>", "bytes": conv_bytes, "ms": conv_ms, "key": "conv"}
     else:
         dom = {"kernel": "build_book_kernel<false>", "bytes": rule_bytes, "ms": rulegen_ms, "key": "rules"}
     achieved = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9

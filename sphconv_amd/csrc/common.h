@@ -44,3 +44,18 @@ static inline int sph_geom_ok(const sph_geom *g)
     if (icol > 0x7fffffffL || ocol > 0x7fffffffL) return 0;
     return 1;
 }
+
+// Workgroups are handed to the 8 XCDs of an MI355X round robin (workgroup i runs on
+// XCD i % 8) and every XCD has its own L2.  Neighbouring tiles share feature rows and
+// index ranges, so each XCD is given one contiguous run of tiles: launch
+// sph_xcd_grid(ntiles) workgroups and map blockIdx.x with sph_xcd_tile(); a result
+// >= ntiles means "no tile, exit".
+#define SPH_NUM_XCD 8
+static inline int sph_xcd_grid(int ntiles) { return sph_div_up(ntiles, SPH_NUM_XCD) * SPH_NUM_XCD; }
+#ifdef __HIPCC__
+__device__ __forceinline__ int sph_xcd_tile(int block, int ntiles)
+{
+    const int per_xcd = (ntiles + SPH_NUM_XCD - 1) / SPH_NUM_XCD;
+    return (block % SPH_NUM_XCD) * per_xcd + block / SPH_NUM_XCD;
+}
+#endif

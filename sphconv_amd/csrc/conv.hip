@@ -1,12 +1,13 @@
 // Gather-GEMM-scatter convolution for gfx950 (wave64, MFMA 16x16 tiles).
 //
-// Forward / dgrad (sph_conv_apply): one workgroup owns SPH_TILE_ROWS consecutive
-// owner rows; wave w owns owner columns [16w, 16w+16).  The tile's pairs arrive
-// as groups of 16 (one kernel offset per group).  Per group a wave gathers the 16
-// feature rows straight into MFMA A-fragments (16 B per lane), multiplies by the
-// pre-packed weight fragment of that offset and adds the 16x16 result into its
-// private columns of an LDS accumulator tile; the tile is written to HBM once,
-// with the epilogue fused.  No atomics, summation order fixed by the book.
+// Forward / dgrad (sph_conv_apply): the tile's pairs arrive as groups of 16 (one
+// kernel offset per group).  Fast kernel (conv_wave_kernel): one wave owns a
+// 128-row tile (x 64 output columns), gathers each group's 16 feature rows straight
+// into MFMA operand registers (16 B per lane), multiplies by the pre-packed weight
+// fragments of that offset and adds the result into its private LDS accumulator
+// tile; the tile is written to HBM once, with the epilogue fused.  No barriers, no
+// atomics, summation order fixed by the book.  conv_apply_kernel is the general
+// fallback for unaligned or very long rows.
 //
 // wgrad (sph_conv_wgrad): a workgroup owns (kernel offset, range of tiles),
 // transposes gathered rows through LDS so that the pair index becomes the MFMA
@@ -184,14 +185,13 @@ __device__ __forceinline__ void acc_add4(uint32_t *p, typename Traits<DT>::acc4 
 }
 
 constexpr int kMetaGroups = 32; // groups whose indices are staged in LDS at a time
-constexpr int kUnroll = 4;      // groups whose fragments are in flight together
 
+// General kernel (any row length and alignment; used when the rows are not a
+// multiple of 16 bytes or longer than 256 bytes): NW waves per tile, wave w owns
+// columns [16w, 16w+16), one group at a time, every wave gathers for itself.
 // The MFMA is issued transposed: D^T[16 owner columns, 16 pairs] = W^T x A^T, so
-// lane l ends up with columns 4*(l/16)..+3 of pair l%16.
-//
-// NSTEP > 0: number of 64-byte steps per gathered row, known at compile time (the
-// fragments of kUnroll groups are then loaded before the first MFMA);
-// NSTEP == 0: any row length, one group at a time.
+// lane l ends up with columns 4*(l/16)..+3 of pair l%16.  NSTEP is always 0 (row
+// length taken from the arguments).
 template <sph_dtype DT, int NW, int NSTEP>
 __global__ __launch_bounds__(NW * kWave) void conv_apply_kernel(ConvArgs a)
 {
@@ -201,13 +201,13 @@ __global__ __launch_bounds__(NW * kWave) void conv_apply_kernel(ConvArgs a)
     extern __shared__ __attribute__((aligned(16))) uint32_t s_acc[]; // [R][LDW]
     __shared__ int s_k[kMetaGroups];
     __shared__ int2 s_meta[kMetaGroups * SPH_GROUP]; // (gathered row, owner row - r0)
-    __shared__ int4v s_afrag[kUnroll * (NSTEP > 0 ? NSTEP : 1) * kWave]; // gathered fragments of one chunk
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    const int tile = blockIdx.x;
+    const int tile = sph_xcd_tile(blockIdx.x, (a.book.rows + R - 1) / R);
     const int r0 = tile * R;
+    if (r0 >= a.book.rows) return; // grid is padded to a multiple of the XCD count
     const int nrows = min(R, a.book.rows - r0);
 
     // each wave clears and later updates only its own 16 columns
@@ -233,67 +233,7 @@ __global__ __launch_bounds__(NW * kWave) void conv_apply_kernel(ConvArgs a)
         for (int i = tid; i < nc; i += NW * kWave) s_k[i] = a.book.grp_k[gb0 + c0 + i];
         __syncthreads();
 
-        if (NSTEP > 0) {
-            // Groups are taken kUnroll at a time.  Each group's 16 rows are gathered by ONE
-            // wave (16 B per lane, already in MFMA operand order) and handed to the other
-            // waves through LDS, so a row crosses the vector memory path once per workgroup
-            // instead of once per wave.  Gathers and weight fragments of the next chunk are
-            // in flight while the current chunk is multiplied.
-            constexpr int NS = NSTEP > 0 ? NSTEP : 1;
-            constexpr int MAXG = (kUnroll + NW - 1) / NW; // groups of a chunk gathered by one wave
-            int4v a_next[MAXG][NS], w_next[kUnroll][NS], w_cur[kUnroll][NS];
-            auto gather_chunk = [&](int g0) {
-#pragma unroll
-                for (int j = 0; j < MAXG; j++) {
-                    const int u = wave + j * NW;
-                    const int in_row = (u < kUnroll && g0 + u < nc) ? s_meta[(g0 + u) * SPH_GROUP + (lane & 15)].x : -1;
-#pragma unroll
-                    for (int st = 0; st < NS; st++) a_next[j][st] = load_a_frag<DT>(a, in_row, st, lane);
-                }
-            };
-            auto weights_chunk = [&](int g0) {
-#pragma unroll
-                for (int u = 0; u < kUnroll; u++) {
-                    const int k = (g0 + u < nc) ? s_k[g0 + u] : 0;
-                    const char *wk = wlane + (long)k * NS * wstep;
-#pragma unroll
-                    for (int st = 0; st < NS; st++) w_next[u][st] = *(const int4v *)(wk + st * wstep);
-                }
-            };
-            gather_chunk(0);
-            weights_chunk(0);
-            for (int g = 0; g < nc; g += kUnroll) {
-#pragma unroll
-                for (int j = 0; j < MAXG; j++) {
-                    const int u = wave + j * NW;
-                    if (u < kUnroll) {
-#pragma unroll
-                        for (int st = 0; st < NS; st++) s_afrag[(u * NS + st) * kWave + lane] = a_next[j][st];
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < kUnroll; u++)
-#pragma unroll
-                    for (int st = 0; st < NS; st++) w_cur[u][st] = w_next[u][st];
-                __syncthreads();
-                if (g + kUnroll < nc) {
-                    gather_chunk(g + kUnroll);
-                    weights_chunk(g + kUnroll);
-                }
-#pragma unroll
-                for (int u = 0; u < kUnroll; u++) {
-                    if (g + u < nc) {
-                        acc4 d = {0, 0, 0, 0};
-#pragma unroll
-                        for (int st = 0; st < NS; st++)
-                            d = mfma_step<DT>(w_cur[u][st], s_afrag[(u * NS + st) * kWave + lane], d);
-                        const int rl = s_meta[(g + u) * SPH_GROUP + (lane & 15)].y;
-                        if (rl >= 0) acc_add4<DT>(&s_acc[rl * LDW + acc_col], d);
-                    }
-                }
-                __syncthreads(); // the fragments are consumed before the next chunk overwrites them
-            }
-        } else {
+        {
             for (int g = 0; g < nc; g++) {
                 const int2 m = s_meta[g * SPH_GROUP + (lane & 15)];
                 const char *wk = wlane + (long)s_k[g] * nsteps * wstep;
@@ -326,6 +266,176 @@ __global__ __launch_bounds__(NW * kWave) void conv_apply_kernel(ConvArgs a)
         for (int i = tid; i < nrows * a.ndim; i += NW * kWave) {
             int row = i / a.ndim, c = i - row * a.ndim;
             out[i] = to_elem<DT>(epilogue_value<DT>(a, s_acc[row * LDW + c], c));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// One wave per tile and per block of 64 output columns.
+//
+// At LiDAR sizes (a few hundred tiles) every workgroup of the grid is resident at
+// once, so the kernel lasts as long as ONE tile's dependent chain; barriers and
+// fragment exchange between waves only lengthen that chain.  Here a wave owns a
+// tile (x 64 columns) outright: it gathers each group's rows once (16 B per lane,
+// already MFMA operand order), holds the offset's weight fragments in registers
+// (re-used while consecutive groups share the offset), and adds into its own LDS
+// accumulator tile.  No barrier, no atomics, summation order = book order.
+// Indices run two blocks ahead, gathers one block ahead, weights one group ahead.
+// ---------------------------------------------------------------------------
+constexpr int kBlk = 4; // groups per pipeline block (4 x 16 index entries = one 64-lane load)
+
+template <sph_dtype DT, int NS, int CT>
+__global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
+{
+    typedef typename Traits<DT>::elem elem;
+    typedef typename Traits<DT>::acc4 acc4;
+    extern __shared__ __attribute__((aligned(16))) uint32_t s_acc[]; // [R][LDW]
+    const int LDW = nwtot * 16 + 4;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;              // block of CT*16 columns
+    const int tile = sph_xcd_tile(blockIdx.x, (a.book.rows + R - 1) / R);
+    const int r0 = tile * R;
+    if (r0 >= a.book.rows) return;
+    const int nrows = min(R, a.book.rows - r0);
+    const int col0 = wave * CT * 16;           // first column of this wave
+
+    for (int i = lane; i < R * CT * 4; i += kWave)
+        *(int4v *)&s_acc[(i / (CT * 4)) * LDW + col0 + (i % (CT * 4)) * 4] = int4v{0, 0, 0, 0};
+
+    const int ngrp = a.book.tile_ngrp[tile];
+    const long gb0 = (long)tile * a.cap;
+    const int32_t *gat = a.book.grp_gather + gb0 * SPH_GROUP;
+    const int32_t *own = a.book.grp_owner + gb0 * SPH_GROUP;
+    const int32_t *gk = a.book.grp_k + gb0;
+    // weight fragment of (offset k, step st, column tile c): k*NS*nwtot + st*nwtot + c  (1 KiB each)
+    const char *wlane = a.wp + ((long)(wave * CT)) * (kWave * 16) + lane * 16;
+    const long wstep = (long)nwtot * (kWave * 16);
+
+    // Every load below is unconditional and straight-line (indices are clamped to
+    // memory that is always allocated, results of invalid slots are discarded by
+    // selects): the compiler can then count outstanding loads exactly and only waits
+    // for the ones an instruction needs.
+    auto load_meta = [&](int g0, int &gi, int &ow, int &kk) {
+        // one load each: lane l holds entry l%16 of group g0 + l/16; lanes 0..3 hold the offsets
+        const int gs = min(g0, a.cap - kBlk); // stay inside this tile's capacity
+        const int g = g0 + (lane >> 4);
+        int vgi = gat[(long)gs * SPH_GROUP + lane];
+        int vow = own[(long)gs * SPH_GROUP + lane] - r0;
+        int vk = gk[gs + (lane & (kBlk - 1))];
+        const bool ok = g < ngrp && gs == g0 && (unsigned)vow < (unsigned)nrows &&
+                        (unsigned)vgi < (unsigned)a.feat_rows;
+        gi = ok ? vgi : -1;
+        ow = ok ? vow : -1;
+        kk = (gs == g0 && g0 + (lane & (kBlk - 1)) < ngrp && (unsigned)vk < (unsigned)a.book.KV) ? vk : 0;
+    };
+    auto load_a = [&](int gi_blk, int4v (&fa)[kBlk][NS]) {
+#pragma unroll
+        for (int u = 0; u < kBlk; u++) {
+            const int in_row = __shfl(gi_blk, u * SPH_GROUP + (lane & 15), kWave);
+            const char *row = a.feat + (long)max(in_row, 0) * a.row_bytes;
+#pragma unroll
+            for (int st = 0; st < NS; st++) {
+                const int off = st * 64 + (lane >> 4) * 16; // rows shorter than 64*NS bytes end early
+                const bool ok = in_row >= 0 && off < a.row_bytes;
+                int4v f = *(const int4v *)(row + (ok ? off : 0));
+                fa[u][st] = ok ? f : int4v{0, 0, 0, 0};
+            }
+        }
+    };
+    auto load_w = [&](int k, int4v (&fw)[NS][CT]) {
+        const char *wk = wlane + (long)k * NS * wstep;
+#pragma unroll
+        for (int st = 0; st < NS; st++)
+#pragma unroll
+            for (int c = 0; c < CT; c++) fw[st][c] = *(const int4v *)(wk + st * wstep + (long)c * (kWave * 16));
+    };
+    auto multiply_add = [&](const int4v (&fw)[NS][CT], const int4v (&fa)[NS], int rl) {
+        // the accumulator rows are requested from LDS before the MFMAs and added after
+        // them, so the LDS round trip hides behind the matrix instructions
+        uint32_t *p = &s_acc[max(rl, 0) * LDW + col0 + (lane >> 4) * 4];
+        acc4 old[CT], d[CT];
+#pragma unroll
+        for (int c = 0; c < CT; c++) {
+            old[c] = *(const acc4 *)(p + c * 16);
+            d[c] = acc4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int st = 0; st < NS; st++)
+#pragma unroll
+            for (int c = 0; c < CT; c++) d[c] = mfma_step<DT>(fw[st][c], fa[st], d[c]);
+        if (rl >= 0) {
+#pragma unroll
+            for (int c = 0; c < CT; c++) *(acc4 *)(p + c * 16) = old[c] + d[c];
+        }
+    };
+
+    // Pipeline: indices run two blocks ahead, gathers one block ahead, weight fragments
+    // three groups ahead (the register set freed by the previous group takes the load).
+    int gi_n, ow_n, k_n;       // indices of the next block
+    int gi_nn, ow_nn, k_nn;    // indices of the block after it
+    int4v a_c[kBlk][NS], a_n[kBlk][NS];
+    int4v w_0[NS][CT], w_1[NS][CT], w_2[NS][CT], w_3[NS][CT]; // fragments for group u of a block live in w_u
+    int ow_c, k_c;
+
+    load_meta(0, gi_n, ow_n, k_n);
+    load_meta(kBlk, gi_nn, ow_nn, k_nn);
+    load_a(gi_n, a_n);
+    load_w(__builtin_amdgcn_readlane(k_n, 0), w_0);
+    load_w(__builtin_amdgcn_readlane(k_n, 1), w_1);
+    load_w(__builtin_amdgcn_readlane(k_n, 2), w_2);
+
+    for (int g0 = 0; g0 < ngrp; g0 += kBlk) {
+#pragma unroll
+        for (int u = 0; u < kBlk; u++)
+#pragma unroll
+            for (int st = 0; st < NS; st++) a_c[u][st] = a_n[u][st];
+        ow_c = ow_n; k_c = k_n;
+        gi_n = gi_nn; ow_n = ow_nn; k_n = k_nn;
+        load_a(gi_n, a_n);
+        load_meta(g0 + 2 * kBlk, gi_nn, ow_nn, k_nn);
+
+        load_w(__builtin_amdgcn_readlane(k_c, 3), w_3);
+        multiply_add(w_0, a_c[0], __shfl(ow_c, 0 * SPH_GROUP + (lane & 15), kWave));
+        load_w(__builtin_amdgcn_readlane(k_n, 0), w_0);
+        multiply_add(w_1, a_c[1], __shfl(ow_c, 1 * SPH_GROUP + (lane & 15), kWave));
+        load_w(__builtin_amdgcn_readlane(k_n, 1), w_1);
+        multiply_add(w_2, a_c[2], __shfl(ow_c, 2 * SPH_GROUP + (lane & 15), kWave));
+        load_w(__builtin_amdgcn_readlane(k_n, 2), w_2);
+        multiply_add(w_3, a_c[3], __shfl(ow_c, 3 * SPH_GROUP + (lane & 15), kWave));
+    }
+
+    // epilogue: this wave's columns of rows [r0, r0+nrows)
+    constexpr int VE = 16 / (int)sizeof(elem);
+    const int ncols = min(CT * 16, a.ndim - col0);
+    if (ncols <= 0) return;
+    elem *out = (elem *)a.out + (long)r0 * a.ndim + col0;
+    const bool plain = DT != SPH_I8 && !a.scale && !a.shift && !a.relu;
+    if (a.aligned_out && ncols % VE == 0) {
+        // lane = (row within a pass, 16-byte chunk of the row): VE accumulators -> one 16-byte store
+        const int cpr = ncols / VE;                 // chunks per row (power of two here)
+        const int ch = lane % cpr, rstep = kWave / cpr;
+        for (int row = lane / cpr; row < nrows; row += rstep) {
+            const uint32_t *src = &s_acc[row * LDW + col0 + ch * VE];
+            union { int4v v; elem e[VE]; } u;
+            if (plain) {
+#pragma unroll
+                for (int j = 0; j < VE; j += 4) {
+                    const float4v f = *(const float4v *)(src + j);
+                    u.e[j] = (elem)f.x; u.e[j + 1] = (elem)f.y; u.e[j + 2] = (elem)f.z; u.e[j + 3] = (elem)f.w;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < VE; j++)
+                    u.e[j] = to_elem<DT>(epilogue_value<DT>(a, src[j], col0 + ch * VE + j));
+            }
+            *(int4v *)(out + (long)row * a.ndim + ch * VE) = u.v;
+        }
+    } else {
+        for (int i = lane; i < nrows * ncols; i += kWave) {
+            int row = i / ncols, c = i - row * ncols;
+            out[(long)row * a.ndim + c] = to_elem<DT>(epilogue_value<DT>(a, s_acc[row * LDW + col0 + c], col0 + c));
         }
     }
 }
@@ -474,22 +584,43 @@ int launch_conv_ns(const ConvArgs &a, int ntiles, hipStream_t st)
     size_t lds = (size_t)R * (NW * 16 + 4) * sizeof(uint32_t);
     int rc = set_lds(conv_apply_kernel<DT, NW, NSTEP>, lds);
     if (rc) return rc;
-    hipLaunchKernelGGL((conv_apply_kernel<DT, NW, NSTEP>), dim3(ntiles), dim3(NW * kWave), lds, st, a);
+    hipLaunchKernelGGL((conv_apply_kernel<DT, NW, NSTEP>), dim3(sph_xcd_grid(ntiles)), dim3(NW * kWave), lds, st, a);
     return sph_check_launch("sph_conv_apply");
+}
+
+template <sph_dtype DT, int NS, int CT>
+int launch_conv_wave(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
+{
+    size_t lds = (size_t)R * (nwtot * 16 + 4) * sizeof(uint32_t);
+    int rc = set_lds(conv_wave_kernel<DT, NS, CT>, lds);
+    if (rc) return rc;
+    const int waves = (nwtot + CT - 1) / CT;
+    hipLaunchKernelGGL((conv_wave_kernel<DT, NS, CT>), dim3(sph_xcd_grid(ntiles)), dim3(waves * kWave), lds, st, a, nwtot);
+    return sph_check_launch("sph_conv_apply");
+}
+
+template <sph_dtype DT, int NS>
+int launch_conv_wave_ct(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
+{
+    switch (nwtot) { // at most two waves per workgroup (launch bound of the kernel)
+    case 1: return launch_conv_wave<DT, NS, 1>(a, nwtot, ntiles, st);
+    case 2: return launch_conv_wave<DT, NS, 2>(a, nwtot, ntiles, st);
+    default: return launch_conv_wave<DT, NS, 4>(a, nwtot, ntiles, st);
+    }
 }
 
 template <sph_dtype DT, int NW>
 int launch_conv(const ConvArgs &a, int ntiles, hipStream_t st)
 {
-    if (a.aligned_in) {
+    if (a.aligned_in && a.feat_rows > 0) {
         switch (a.nsteps) {
-        case 1: return launch_conv_ns<DT, NW, 1>(a, ntiles, st);
-        case 2: return launch_conv_ns<DT, NW, 2>(a, ntiles, st);
-        case 4: return launch_conv_ns<DT, NW, 4>(a, ntiles, st);
+        case 1: return launch_conv_wave_ct<DT, 1>(a, NW, ntiles, st);
+        case 2: return launch_conv_wave_ct<DT, 2>(a, NW, ntiles, st);
+        case 4: return launch_conv_wave_ct<DT, 4>(a, NW, ntiles, st);
         default: break;
         }
     }
-    return launch_conv_ns<DT, NW, 0>(a, ntiles, st);
+    return launch_conv_ns<DT, NW, 0>(a, ntiles, st); // rows not a multiple of 16 bytes, or more than 256 bytes
 }
 
 template <sph_dtype DT>

@@ -208,10 +208,11 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     __shared__ int s_tmp, s_flag;
 
     const int tid = threadIdx.x;
-    const int tile = blockIdx.x;
+    const int tile = sph_xcd_tile(blockIdx.x, (a.q_rows + R - 1) / R);
     const int KV = a.cv.K0 * a.cv.K1 * a.cv.K2;
     const int K01 = a.cv.K0 * a.cv.K1;
     const int r0 = tile * R;
+    if (r0 >= a.q_rows) return; // grid is padded to a multiple of the XCD count
     const int r1 = min(r0 + R, a.q_rows);
     const int nrows = r1 - r0;
     const int q_ncol = a.B * a.Q.n0 * a.Q.n1;
@@ -635,9 +636,9 @@ SPH_EXPORT int sph_rules_build(const int32_t *z_idx, const int32_t *z_ptr, int i
     const size_t lds = (size_t)R * KV * sizeof(int32_t);
     hipStream_t st = (hipStream_t)stream;
     if (!transposed)
-        hipLaunchKernelGGL(build_book_kernel<false>, dim3(nt), dim3(kThreads), lds, st, a);
+        hipLaunchKernelGGL(build_book_kernel<false>, dim3(sph_xcd_grid(nt)), dim3(kThreads), lds, st, a);
     else
-        hipLaunchKernelGGL(build_book_kernel<true>, dim3(nt), dim3(kThreads), lds, st, a);
+        hipLaunchKernelGGL(build_book_kernel<true>, dim3(sph_xcd_grid(nt)), dim3(kThreads), lds, st, a);
     return sph_check_launch("sph_rules_build");
 }
 
