@@ -301,9 +301,6 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
     const int nrows = min(R, a.book.rows - r0);
     const int col0 = wave * CT * 16;           // first column of this wave
 
-    for (int i = lane; i < R * CT * 4; i += kWave)
-        *(int4v *)&s_acc[(i / (CT * 4)) * LDW + col0 + (i % (CT * 4)) * 4] = int4v{0, 0, 0, 0};
-
     const int ngrp = a.book.tile_ngrp[tile];
     const long gb0 = (long)tile * a.cap;
     const int32_t *gat = a.book.grp_gather + gb0 * SPH_GROUP;
@@ -381,6 +378,9 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
 
     load_meta(0, gi_n, ow_n, k_n);
     load_meta(kBlk, gi_nn, ow_nn, k_nn);
+    // clear the accumulator tile while the first indices are on their way
+    for (int i = lane; i < R * CT * 4; i += kWave)
+        *(int4v *)&s_acc[(i / (CT * 4)) * LDW + col0 + (i % (CT * 4)) * 4] = int4v{0, 0, 0, 0};
     load_a(gi_n, a_n);
     load_w(__builtin_amdgcn_readlane(k_n, 0), w_0);
     load_w(__builtin_amdgcn_readlane(k_n, 1), w_1);
@@ -416,21 +416,39 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
         // lane = (row within a pass, 16-byte chunk of the row): VE accumulators -> one 16-byte store
         const int cpr = ncols / VE;                 // chunks per row (power of two here)
         const int ch = lane % cpr, rstep = kWave / cpr;
-        for (int row = lane / cpr; row < nrows; row += rstep) {
-            const uint32_t *src = &s_acc[row * LDW + col0 + ch * VE];
-            union { int4v v; elem e[VE]; } u;
-            if (plain) {
+        if (plain) {
+            // four rows per pass: their LDS reads are all issued before the first conversion
+            constexpr int UR = 4;
+            for (int row0 = lane / cpr; row0 < nrows; row0 += UR * rstep) {
+                float4v f[UR][VE / 4];
 #pragma unroll
-                for (int j = 0; j < VE; j += 4) {
-                    const float4v f = *(const float4v *)(src + j);
-                    u.e[j] = (elem)f.x; u.e[j + 1] = (elem)f.y; u.e[j + 2] = (elem)f.z; u.e[j + 3] = (elem)f.w;
+                for (int q = 0; q < UR; q++) {
+                    const int row = min(row0 + q * rstep, nrows - 1);
+#pragma unroll
+                    for (int j = 0; j < VE / 4; j++)
+                        f[q][j] = *(const float4v *)&s_acc[row * LDW + col0 + ch * VE + j * 4];
                 }
-            } else {
+#pragma unroll
+                for (int q = 0; q < UR; q++) {
+                    const int row = row0 + q * rstep;
+                    union { int4v v; elem e[VE]; } u;
+#pragma unroll
+                    for (int j = 0; j < VE / 4; j++) {
+                        u.e[4 * j] = (elem)f[q][j].x; u.e[4 * j + 1] = (elem)f[q][j].y;
+                        u.e[4 * j + 2] = (elem)f[q][j].z; u.e[4 * j + 3] = (elem)f[q][j].w;
+                    }
+                    if (row < nrows) *(int4v *)(out + (long)row * a.ndim + ch * VE) = u.v;
+                }
+            }
+        } else {
+            for (int row = lane / cpr; row < nrows; row += rstep) {
+                const uint32_t *src = &s_acc[row * LDW + col0 + ch * VE];
+                union { int4v v; elem e[VE]; } u;
 #pragma unroll
                 for (int j = 0; j < VE; j++)
                     u.e[j] = to_elem<DT>(epilogue_value<DT>(a, src[j], col0 + ch * VE + j));
+                *(int4v *)(out + (long)row * a.ndim + ch * VE) = u.v;
             }
-            *(int4v *)(out + (long)row * a.ndim + ch * VE) = u.v;
         }
     } else {
         for (int i = lane; i < nrows * ncols; i += kWave) {
