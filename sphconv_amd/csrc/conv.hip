@@ -314,19 +314,28 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
     // memory that is always allocated, results of invalid slots are discarded by
     // selects): the compiler can then count outstanding loads exactly and only waits
     // for the ones an instruction needs.
+    // Index loads return raw values; they are validated (finish_meta) only when the block
+    // is about to be used, one or two blocks later -- touching a loaded value earlier
+    // would make the wave wait for it, and with it for every load issued before.
     auto load_meta = [&](int g0, int &gi, int &ow, int &kk) {
         // one load each: lane l holds entry l%16 of group g0 + l/16; lanes 0..3 hold the offsets
         const int gs = min(g0, a.cap - kBlk); // stay inside this tile's capacity
-        const int g = g0 + (lane >> 4);
-        int vgi = gat[(long)gs * SPH_GROUP + lane];
-        int vow = own[(long)gs * SPH_GROUP + lane] - r0;
-        int vk = gk[gs + (lane & (kBlk - 1))];
-        const bool ok = g < ngrp && gs == g0 && (unsigned)vow < (unsigned)nrows &&
-                        (unsigned)vgi < (unsigned)a.feat_rows;
-        gi = ok ? vgi : -1;
-        ow = ok ? vow : -1;
-        kk = (gs == g0 && g0 + (lane & (kBlk - 1)) < ngrp && (unsigned)vk < (unsigned)a.book.KV) ? vk : 0;
+        gi = gat[(long)gs * SPH_GROUP + lane];
+        ow = own[(long)gs * SPH_GROUP + lane];
+        kk = gk[gs + (lane & (kBlk - 1))];
     };
+    auto finish_meta = [&](int g0, int &gi, int &ow, int &kk) {
+        const bool inside = g0 <= a.cap - kBlk;
+        const int g = g0 + (lane >> 4);
+        const int vow = ow - r0;
+        const bool ok = inside && g < ngrp && (unsigned)vow < (unsigned)nrows && (unsigned)gi < (unsigned)a.feat_rows;
+        gi = ok ? gi : -1;
+        ow = ok ? vow : -1;
+        kk = (inside && g0 + (lane & (kBlk - 1)) < ngrp && (unsigned)kk < (unsigned)a.book.KV) ? kk : 0;
+    };
+    // Gathers only load (from an address clamped into the feature array); slots that hold
+    // no pair and the tail of rows shorter than the step are zeroed when the fragment is
+    // used, not here -- a select on the loaded value would stall the wave on the load.
     auto load_a = [&](int gi_blk, int4v (&fa)[kBlk][NS]) {
 #pragma unroll
         for (int u = 0; u < kBlk; u++) {
@@ -334,10 +343,8 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
             const char *row = a.feat + (long)max(in_row, 0) * a.row_bytes;
 #pragma unroll
             for (int st = 0; st < NS; st++) {
-                const int off = st * 64 + (lane >> 4) * 16; // rows shorter than 64*NS bytes end early
-                const bool ok = in_row >= 0 && off < a.row_bytes;
-                int4v f = *(const int4v *)(row + (ok ? off : 0));
-                fa[u][st] = ok ? f : int4v{0, 0, 0, 0};
+                const int off = st * 64 + (lane >> 4) * 16;
+                fa[u][st] = *(const int4v *)(row + (off < a.row_bytes ? off : 0));
             }
         }
     };
@@ -348,24 +355,36 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
 #pragma unroll
             for (int c = 0; c < CT; c++) fw[st][c] = *(const int4v *)(wk + st * wstep + (long)c * (kWave * 16));
     };
+    const bool short_rows = a.row_bytes < NS * 64; // the last step reads past the row: mask it
     auto multiply_add = [&](const int4v (&fw)[NS][CT], const int4v (&fa)[NS], int rl) {
-        // the accumulator rows are requested from LDS before the MFMAs and added after
-        // them, so the LDS round trip hides behind the matrix instructions
-        uint32_t *p = &s_acc[max(rl, 0) * LDW + col0 + (lane >> 4) * 4];
+        // The accumulator rows are requested from LDS before the MFMAs and added after
+        // them, so the LDS round trip hides behind the matrix instructions.  Padding
+        // slots (rl < 0) multiply whatever row 0 holds and add into a scratch row behind
+        // the tile: no branch, no select, and nothing real is touched.
+        uint32_t *p = &s_acc[(rl >= 0 ? rl : R) * LDW + col0 + (lane >> 4) * 4];
         acc4 old[CT], d[CT];
 #pragma unroll
         for (int c = 0; c < CT; c++) {
             old[c] = *(const acc4 *)(p + c * 16);
             d[c] = acc4{0, 0, 0, 0};
         }
+        __builtin_amdgcn_sched_barrier(0);
+        if (short_rows) { // uniform; e.g. 4 fp32 channels = 16 of the step's 64 bytes
 #pragma unroll
-        for (int st = 0; st < NS; st++)
+            for (int st = 0; st < NS; st++) {
+                const bool live = st * 64 + (lane >> 4) * 16 < a.row_bytes;
+                const int4v x = live ? fa[st] : int4v{0, 0, 0, 0};
 #pragma unroll
-            for (int c = 0; c < CT; c++) d[c] = mfma_step<DT>(fw[st][c], fa[st], d[c]);
-        if (rl >= 0) {
+                for (int c = 0; c < CT; c++) d[c] = mfma_step<DT>(fw[st][c], x, d[c]);
+            }
+        } else {
 #pragma unroll
-            for (int c = 0; c < CT; c++) *(acc4 *)(p + c * 16) = old[c] + d[c];
+            for (int st = 0; st < NS; st++)
+#pragma unroll
+                for (int c = 0; c < CT; c++) d[c] = mfma_step<DT>(fw[st][c], fa[st], d[c]);
         }
+#pragma unroll
+        for (int c = 0; c < CT; c++) *(acc4 *)(p + c * 16) = old[c] + d[c];
     };
 
     // Pipeline: indices run two blocks ahead, gathers one block ahead, weight fragments
@@ -378,9 +397,10 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
 
     load_meta(0, gi_n, ow_n, k_n);
     load_meta(kBlk, gi_nn, ow_nn, k_nn);
-    // clear the accumulator tile while the first indices are on their way
-    for (int i = lane; i < R * CT * 4; i += kWave)
+    // clear the accumulator tile (and the scratch row) while the first indices are on their way
+    for (int i = lane; i < (R + 1) * CT * 4; i += kWave)
         *(int4v *)&s_acc[(i / (CT * 4)) * LDW + col0 + (i % (CT * 4)) * 4] = int4v{0, 0, 0, 0};
+    finish_meta(0, gi_n, ow_n, k_n);
     load_a(gi_n, a_n);
     load_w(__builtin_amdgcn_readlane(k_n, 0), w_0);
     load_w(__builtin_amdgcn_readlane(k_n, 1), w_1);
@@ -393,16 +413,28 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
             for (int st = 0; st < NS; st++) a_c[u][st] = a_n[u][st];
         ow_c = ow_n; k_c = k_n;
         gi_n = gi_nn; ow_n = ow_nn; k_n = k_nn;
+        finish_meta(g0 + kBlk, gi_n, ow_n, k_n);   // loaded one block ago
+        // Loads complete in issue order: the weight fragment needed at the end of this
+        // block goes first, so that waiting for it does not also wait for the gathers.
+        // Scheduling barriers keep the compiler from moving a prefetch down to its use.
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(__builtin_amdgcn_readlane(k_c, 3), w_3);
+        __builtin_amdgcn_sched_barrier(0);
         load_a(gi_n, a_n);
         load_meta(g0 + 2 * kBlk, gi_nn, ow_nn, k_nn);
-
-        load_w(__builtin_amdgcn_readlane(k_c, 3), w_3);
+        __builtin_amdgcn_sched_barrier(0);
         multiply_add(w_0, a_c[0], __shfl(ow_c, 0 * SPH_GROUP + (lane & 15), kWave));
+        __builtin_amdgcn_sched_barrier(0);
         load_w(__builtin_amdgcn_readlane(k_n, 0), w_0);
+        __builtin_amdgcn_sched_barrier(0);
         multiply_add(w_1, a_c[1], __shfl(ow_c, 1 * SPH_GROUP + (lane & 15), kWave));
+        __builtin_amdgcn_sched_barrier(0);
         load_w(__builtin_amdgcn_readlane(k_n, 1), w_1);
+        __builtin_amdgcn_sched_barrier(0);
         multiply_add(w_2, a_c[2], __shfl(ow_c, 2 * SPH_GROUP + (lane & 15), kWave));
+        __builtin_amdgcn_sched_barrier(0);
         load_w(__builtin_amdgcn_readlane(k_n, 2), w_2);
+        __builtin_amdgcn_sched_barrier(0);
         multiply_add(w_3, a_c[3], __shfl(ow_c, 3 * SPH_GROUP + (lane & 15), kWave));
     }
 
@@ -609,7 +641,7 @@ int launch_conv_ns(const ConvArgs &a, int ntiles, hipStream_t st)
 template <sph_dtype DT, int NS, int CT>
 int launch_conv_wave(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
 {
-    size_t lds = (size_t)R * (nwtot * 16 + 4) * sizeof(uint32_t);
+    size_t lds = (size_t)(R + 1) * (nwtot * 16 + 4) * sizeof(uint32_t); // + scratch row
     int rc = set_lds(conv_wave_kernel<DT, NS, CT>, lds);
     if (rc) return rc;
     const int waves = (nwtot + CT - 1) / CT;
