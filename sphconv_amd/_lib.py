@@ -110,7 +110,8 @@ def ptr(t):
 
 
 def stream():
-    return torch.cuda.current_stream().cuda_stream
+    """Raw handle of torch's current HIP stream on the current device."""
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
 
 
 def make_geom(batch, in_shape, out_shape, kernel, stride, padding, dilation=(1, 1, 1)) -> Geom:

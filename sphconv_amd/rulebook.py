@@ -15,7 +15,11 @@ from . import _lib as L
 
 
 class _Buffers:
-    """Device arrays of one book (forward or transposed)."""
+    """Device arrays of one book (forward or transposed), carved out of ONE allocation
+    (a single caching-allocator call per book); the named tensors are views made on
+    first access."""
+
+    _FIELDS = ("tile_ngrp", "tile_koff", "grp_k", "grp_gather", "grp_owner")
 
     def __init__(self, rows: int, kv: int, device):
         lib = L.lib()
@@ -23,16 +27,35 @@ class _Buffers:
         self.ntiles = lib.sph_book_tiles(self.rows)
         self.cap = lib.sph_book_cap(self.kv)
         nt = max(self.ntiles, 1)
-        i32 = dict(dtype=torch.int32, device=device)
-        self.tile_ngrp = torch.empty(nt, **i32)
-        self.tile_koff = torch.empty((nt, self.kv + 1), dtype=torch.int16, device=device)
-        self.grp_k = torch.empty(nt * self.cap, **i32)
-        self.grp_gather = torch.empty(nt * self.cap * L.GROUP, **i32)
-        self.grp_owner = torch.empty(nt * self.cap * L.GROUP, **i32)
+        sizes = (nt * 4, nt * (self.kv + 1) * 2, nt * self.cap * 4, nt * self.cap * L.GROUP * 4,
+                 nt * self.cap * L.GROUP * 4)
+        self._off = []
+        total = 0
+        for sz in sizes:
+            self._off.append(total)
+            total += (sz + 255) & ~255
+        self._sizes = sizes
+        self.storage = torch.empty(total, dtype=torch.uint8, device=device)
+        base = self.storage.data_ptr()
+        self._struct = L.Book(*(base + o for o in self._off), self.rows, self.kv)
+        self._views = {}
 
     def struct(self) -> L.Book:
-        return L.Book(L.ptr(self.tile_ngrp), L.ptr(self.tile_koff), L.ptr(self.grp_k),
-                      L.ptr(self.grp_gather), L.ptr(self.grp_owner), self.rows, self.kv)
+        return self._struct
+
+    def __getattr__(self, name):
+        # views of the single allocation, typed and shaped like the C arrays
+        if name in _Buffers._FIELDS:
+            v = self._views.get(name)
+            if v is None:
+                i = _Buffers._FIELDS.index(name)
+                raw = self.storage[self._off[i]:self._off[i] + self._sizes[i]]
+                v = raw.view(torch.int16 if name == "tile_koff" else torch.int32)
+                if name == "tile_koff":
+                    v = v.view(max(self.ntiles, 1), self.kv + 1)
+                self._views[name] = v
+            return v
+        raise AttributeError(name)
 
     def num_pairs(self) -> int:
         """Total pairs held (synchronises)."""
@@ -76,9 +99,11 @@ class RuleBook:
         rows = self.in_rows if transposed else self.out_rows
         buf = _Buffers(rows, self.kv, self.z_ptr.device)
         g, b = self.geom(), buf.struct()
-        L.check(L.lib().sph_rules_build(L.ptr(self.z_idx), L.ptr(self.z_ptr), self.in_rows,
-                                        L.ptr(self.oz_idx), L.ptr(self.oz_ptr), self.out_rows,
-                                        C.byref(g), int(transposed), C.byref(b), L.stream()))
+        rc = L.lib().sph_rules_build(self.z_idx.data_ptr(), self.z_ptr.data_ptr(), self.in_rows,
+                                     self.oz_idx.data_ptr(), self.oz_ptr.data_ptr(), self.out_rows,
+                                     C.byref(g), int(transposed), C.byref(b), L.stream())
+        if rc:
+            L.check(rc)
         return buf
 
     @classmethod
@@ -208,3 +233,5 @@ def _check_index_tensors(z_idx, z_ptr, batch, shape):
         raise L.SphconvError("z_ptr must be [B,S0,S1] = %s, got %s" % (want, tuple(z_ptr.shape)))
     if not (z_idx.is_contiguous() and z_ptr.is_contiguous()):
         raise L.SphconvError("z_idx and z_ptr must be contiguous")
+    if not (z_idx.is_cuda and z_ptr.is_cuda):
+        raise L.SphconvError("z_idx and z_ptr must be GPU tensors")

@@ -49,14 +49,24 @@ def _as_book(rules, rule_size, in_rows: int, out_rows: int) -> RuleBook:
     return RuleBook.from_padded(rules, rule_size, in_rows, out_rows)
 
 
+_NO_EPILOGUE = L.Epilogue(None, None, 0)
+
+
 def _apply(feature, packed, kdim, ndim, buffers, scale=None, shift=None, relu=False, out_dtype=None):
-    feature = feature.contiguous()
+    if not feature.is_contiguous():
+        feature = feature.contiguous()
+    if not feature.is_cuda:
+        raise L.SphconvError("expected a GPU tensor, got device %s" % feature.device)
     out = torch.empty((buffers.rows, ndim), dtype=out_dtype or feature.dtype, device=feature.device)
-    epi = L.Epilogue(L.ptr(scale), L.ptr(shift), int(bool(relu)))
-    b = buffers.struct()
-    L.check(L.lib().sph_conv_apply(L.dtype_code(feature.dtype), L.ptr(feature), int(feature.shape[0]),
-                                   int(kdim), L.ptr(packed), int(ndim), C.byref(b), C.byref(epi),
-                                   L.ptr(out), L.stream()))
+    if scale is None and shift is None and not relu:
+        epi = _NO_EPILOGUE
+    else:
+        epi = L.Epilogue(L.ptr(scale), L.ptr(shift), int(bool(relu)))
+    rc = L.lib().sph_conv_apply(L.dtype_code(feature.dtype), feature.data_ptr(), feature.shape[0], kdim,
+                                packed.data_ptr(), ndim, C.byref(buffers.struct()), C.byref(epi),
+                                out.data_ptr(), L.stream())
+    if rc:
+        L.check(rc)
     return out
 
 
