@@ -497,6 +497,8 @@ struct WgradArgs {
     sph_book book;
     int cap, ntiles, nchunk;
     float *partial;
+    int *flags;      // wave kernel: one per partial slot, 1 = the slot was written
+    int nslots;
 };
 
 constexpr int kWgThreads = 256;
@@ -601,6 +603,311 @@ __global__ void wgrad_reduce_kernel(const float *partial, int KV, int nchunk, in
     dw[i] = (typename Traits<DT>::elem)s;
 }
 
+// ---------------------------------------------------------------------------
+// wgrad, fast path (rows are whole 16-byte chunks).
+//
+// Work item = (offset k, chunk of 64 tiles, slice of 64 groups of that chunk's
+// groups at k, 64x64 block of [iC,oC]).  A chunk holds at most 64*8 groups per
+// offset, so 8 slices always cover it; slices beyond the chunk's real group count
+// exit at once (a submanifold book has 8 groups per tile at the centre offset and
+// about one elsewhere: slicing by groups, not tiles, is what balances the grid).
+// The four waves of the workgroup take the slice's batches (2 groups = 32 pairs)
+// round robin and never synchronise until the end: a wave gathers the 32 feature
+// rows and 32 d_out rows with 16-byte loads into its own LDS area in natural
+// [pair][channel] order, and reads MFMA operands with the pair index as the K
+// dimension through transposing LDS reads (16-bit types) or strided 4-byte reads
+// (fp32).  The [64,64] block lives in registers; the workgroup's four blocks are
+// summed through LDS into one fp32 partial, and wgrad_slot_reduce_kernel adds
+// the written slots in a fixed order.
+// ---------------------------------------------------------------------------
+constexpr int kWsTiles = 64;   // tiles per chunk (one lane each)
+constexpr int kWsSlice = 64;   // groups per slice
+constexpr int kWsSlices = 4;   // workgroups per (offset, chunk): workgroup h takes slices h, h+4
+constexpr int kWsBlock = 64;   // channels per block side
+
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+// MFMA operand of 16 channels x one batch of pairs from a staging area laid out
+// [pair][channel], row stride rs bytes.  16-bit types: lane (m = lane%16, q = lane/16)
+// receives pairs 8q..8q+7 of channel m through two transposing reads (element j of lane
+// 4a+b = the b-th element at the address given by lane a+4j of the same 16 lanes).
+// fp32: component j of lane (m, q) = pair 4j+q of channel m.
+template <sph_dtype DT>
+__device__ __forceinline__ int wgrad_frag_offset(int rs, int lane)
+{
+    if constexpr (sizeof(typename Traits<DT>::elem) == 2) {
+        const int s = lane & 15, q = lane >> 4;
+        return (8 * q + (s >> 2)) * rs + 4 * (s & 3) * 2;
+    } else {
+        return (lane >> 4) * rs + (lane & 15) * 4;
+    }
+}
+template <sph_dtype DT>
+__device__ __forceinline__ int4v wgrad_frag(const char *p, int rs)
+{
+    if constexpr (sizeof(typename Traits<DT>::elem) == 2) {
+        typedef __attribute__((address_space(3))) short4v lds_s4;
+        short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4 *)p);
+        short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4 *)(p + 4 * rs));
+        union { struct { short4v l, h; } s; int4v v; } u;
+        u.s.l = lo; u.s.h = hi;
+        return u.v;
+    } else {
+        union { float f[4]; int4v v; } u;
+#pragma unroll
+        for (int j = 0; j < 4; j++) u.f[j] = *(const float *)(p + 4 * j * rs);
+        return u.v;
+    }
+}
+
+template <sph_dtype DT, int MI, int NI>
+__global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
+{
+    typedef typename Traits<DT>::elem elem;
+    constexpr int E = (int)sizeof(elem);
+    constexpr int GPB = E == 2 ? 2 : 1;                // groups per batch: one MFMA super step of 32 or 16 pairs
+    constexpr int PB = GPB * SPH_GROUP;                // pairs per batch
+    // MI, NI: 16-channel tiles of the block's two sides (1, 2 or 4; narrower blocks are zero padded).
+    // A batch of rows of MI tiles is MI 16-byte loads per lane.
+    extern __shared__ __attribute__((aligned(16))) char s_raw[];
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int KV = a.book.KV;
+    // Work items u = chunk*KV + k are dealt to the XCDs in contiguous runs (workgroups go to
+    // the XCDs round robin): the offsets of one chunk gather the same ~2 MiB of rows, which
+    // then stay in that XCD's L2.  The slice index is slowest, so that the first slices --
+    // often the only ones with work -- spread over all XCDs and start first.
+    const int items = KV * a.nchunk, items_grid = (items + SPH_NUM_XCD - 1) / SPH_NUM_XCD * SPH_NUM_XCD;
+    const int h = blockIdx.x / items_grid;
+    const int u = sph_xcd_tile(blockIdx.x - h * items_grid, items);
+    if (u >= items) return;
+    const int chunk = u / KV, k = u - chunk * KV;
+    const int sbn = (a.oC + kWsBlock - 1) / kWsBlock;
+    const int ci0 = (blockIdx.y / sbn) * kWsBlock, co0 = (blockIdx.y % sbn) * kWsBlock;
+    const int cA = min(kWsBlock, a.iC - ci0), cG = min(kWsBlock, a.oC - co0);
+    const int slot = (k * a.nchunk + chunk) * kWsSlices + h;
+
+    // groups of this offset in the chunk's tiles: lane = tile, prefix sums over the wave
+    const int t0 = chunk * kWsTiles;
+    int g0 = 0, n = 0;
+    if (t0 + lane < a.ntiles) {
+        const unsigned short *ko = a.book.tile_koff + (long)(t0 + lane) * (KV + 1) + k;
+        g0 = min((int)ko[0], a.cap);
+        n = min(max((int)ko[1] - g0, 0), min(a.cap - g0, R / SPH_GROUP));
+    }
+    int incl = n;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        int v = __shfl_up(incl, d, kWave);
+        if (lane >= d) incl += v;
+    }
+    const int total = __shfl(incl, kWave - 1, kWave);
+    if (h * kWsSlice >= total) {
+        if (tid == 0 && blockIdx.y == 0) a.flags[slot] = 0;
+        return;
+    }
+
+    // wave-private staging: feature rows then d_out rows, [pair][channels + 16 bytes]
+    constexpr int rsA = MI * 16 * E + 16, rsG = NI * 16 * E + 16;
+    const int cprA = cA * E / 16, cprG = cG * E / 16;      // real 16-byte chunks per row
+    char *xa = s_raw + (size_t)wave * PB * (rsA + rsG);
+    char *xg = xa + PB * rsA;
+    for (int i = lane; i < PB * (rsA + rsG) / 16; i += kWave) ((int4v *)xa)[i] = int4v{0, 0, 0, 0};
+
+    float4v acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < NI; j++) acc[i][j] = float4v{0, 0, 0, 0};
+
+    // Per-lane constants of the row copies: which pair and 16-byte chunk each of the lane's
+    // loads moves, its offset in the source row and in the staging area (-1: none).
+    int pairA[MI], srcA[MI], dstA[MI], pairG[NI], srcG[NI], dstG[NI];
+#pragma unroll
+    for (int it = 0; it < MI; it++) {
+        const int i = it * kWave + lane;
+        const int pa = i / cprA, ca = i - pa * cprA;
+        pairA[it] = min(pa, PB - 1); srcA[it] = ci0 * E + ca * 16; dstA[it] = pa < PB ? pa * rsA + ca * 16 : -1;
+    }
+#pragma unroll
+    for (int it = 0; it < NI; it++) {
+        const int i = it * kWave + lane;
+        const int pg = i / cprG, cg = i - pg * cprG;
+        pairG[it] = min(pg, PB - 1); srcG[it] = co0 * E + cg * 16; dstG[it] = pg < PB ? pg * rsG + cg * 16 : -1;
+    }
+    const unsigned strideA = a.iC * E, strideG = a.oC * E;   // arrays are below 4 GiB (checked by the launcher)
+
+    // Book slot of every group of a slice: lane l looks up flattened group s0+l (the tile
+    // whose prefix range holds it, by binary search over the tile lanes) once per slice.
+    const long slot_max = (long)a.ntiles * a.cap * SPH_GROUP - 1;
+    auto slot_bases = [&](int s0) -> int {
+        const int f = s0 + lane;
+        int lo = 0;
+#pragma unroll
+        for (int step = kWave / 2; step >= 1; step >>= 1) {
+            const int v = __shfl(incl, lo + step - 1, kWave);
+            if (v <= f) lo += step;
+        }
+        lo = min(lo, kWave - 1);
+        const int g = __shfl(g0, lo, kWave) + f - (__shfl(incl, lo, kWave) - __shfl(n, lo, kWave));
+        const long sl = ((long)(t0 + lo) * a.cap + g) * SPH_GROUP;
+        return (int)min(max(sl, 0L), slot_max - (SPH_GROUP - 1));   // ntiles*cap*16 fits 31 bits (checked by the launcher)
+    };
+    // Book entries of batch b of the slice: lane l < 32 loads the gathered (input) row of pair
+    // l%PB, lane 32+l its owner (output) row.  The load is unconditional; the value is only
+    // looked at once all of the wave's index loads are on their way.
+    auto load_idx = [&](int bases, int s0, int s1, int b, bool &valid) -> int {
+        const int pr = lane & (PB - 1);
+        const int fl = GPB * b + (pr >> 4);                 // group within the slice
+        valid = s0 + fl < s1;
+        const int base = __shfl(bases, fl & (kWave - 1), kWave);
+        return (lane < 32 ? a.book.grp_gather : a.book.grp_owner)[base + (pr & 15)];
+    };
+    // Row loads are unconditional (clamped to row 0; in_rows and out_rows are positive here)
+    // so that several batches stay in flight; slots without a pair are zeroed when the rows
+    // are staged.  Returns the mask of pairs that exist.
+    auto gather = [&](int idx, int4v (&ra)[MI], int4v (&rg)[NI]) -> unsigned {
+        const int other = __shfl_xor(idx, 32, kWave);
+        const unsigned ok = (unsigned)__ballot(idx >= 0 && other >= 0);
+#pragma unroll
+        for (int it = 0; it < MI; it++) {
+            const int row = max(__shfl(idx, pairA[it], kWave), 0);
+            ra[it] = *(const int4v *)(a.feat + ((unsigned)row * strideA + (unsigned)srcA[it]));
+        }
+#pragma unroll
+        for (int it = 0; it < NI; it++) {
+            const int orow = max(__shfl(idx, 32 + pairG[it], kWave), 0);
+            rg[it] = *(const int4v *)(a.dout + ((unsigned)orow * strideG + (unsigned)srcG[it]));
+        }
+        return ok;
+    };
+    auto stage = [&](unsigned ok, const int4v (&ra)[MI], const int4v (&rg)[NI]) {
+#pragma unroll
+        for (int it = 0; it < MI; it++)
+            if (dstA[it] >= 0) *(int4v *)(xa + dstA[it]) = ((ok >> pairA[it]) & 1) ? ra[it] : int4v{0, 0, 0, 0};
+#pragma unroll
+        for (int it = 0; it < NI; it++)
+            if (dstG[it] >= 0) *(int4v *)(xg + dstG[it]) = ((ok >> pairG[it]) & 1) ? rg[it] : int4v{0, 0, 0, 0};
+    };
+    const char *fragA = xa + wgrad_frag_offset<DT>(rsA, lane), *fragG = xg + wgrad_frag_offset<DT>(rsG, lane);
+    auto multiply = [&]() {
+        int4v fa[MI], fb[NI];
+#pragma unroll
+        for (int i = 0; i < MI; i++) fa[i] = wgrad_frag<DT>(fragA + i * 16 * E, rsA);
+#pragma unroll
+        for (int i = 0; i < NI; i++) fb[i] = wgrad_frag<DT>(fragG + i * 16 * E, rsG);
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int j = 0; j < NI; j++) acc[i][j] = mfma_step<DT>(fa[i], fb[j], acc[i][j]);
+    };
+
+    // Per slice, this wave owns batches wave, wave+4, ... (at most NB).  All their index
+    // entries are requested at once; then the rows run DEPTH-1 batches ahead of their
+    // staging through DEPTH register sets, and staging runs one batch ahead of the MFMAs.
+    // The single staging area is safe because LDS operations of a wave execute in order.
+    constexpr int NB = kWsSlice / GPB / 4;
+    constexpr int DEPTH = 3;
+    for (int s0 = h * kWsSlice; s0 < total; s0 += kWsSlices * kWsSlice) {
+        const int s1 = min(total, s0 + kWsSlice);
+        const int nbatch = (s1 - s0 + GPB - 1) / GPB;
+        const int bases = slot_bases(s0);
+        int idx[NB];
+        bool valid[NB];
+#pragma unroll
+        for (int j = 0; j < NB; j++) idx[j] = load_idx(bases, s0, s1, wave + 4 * j, valid[j]);
+#pragma unroll
+        for (int j = 0; j < NB; j++)
+            idx[j] = (valid[j] && (unsigned)idx[j] < (unsigned)(lane < 32 ? a.in_rows : a.out_rows)) ? idx[j] : -1;
+        int4v ra[DEPTH][MI], rg[DEPTH][NI];
+        unsigned ok[DEPTH];
+#pragma unroll
+        for (int j = 0; j < DEPTH - 1; j++)
+            if (j < NB) ok[j] = gather(idx[j], ra[j], rg[j]);
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+            if (wave + 4 * j < nbatch) {     // wave-uniform
+                if (j + DEPTH - 1 < NB)
+                    ok[(j + DEPTH - 1) % DEPTH] = gather(idx[j + DEPTH - 1], ra[(j + DEPTH - 1) % DEPTH], rg[(j + DEPTH - 1) % DEPTH]);
+                if (j > 0) multiply();            // batch j-1, from LDS
+                asm volatile("" ::: "memory");    // keep the staging writes behind the transposing reads
+                stage(ok[j % DEPTH], ra[j % DEPTH], rg[j % DEPTH]);
+                asm volatile("" ::: "memory");
+            }
+        }
+        if (wave < nbatch) multiply();            // the last staged batch
+    }
+
+    // Sum the four waves' blocks through LDS (over the staging areas), pairwise: (0+2, 1+3),
+    // then (0+1).  The partial is stored in accumulator order -- tile (i,j), lane, 4 values:
+    // element [16i + 4(lane/16) + r][16j + lane%16] -- as 16-byte stores; the reduction kernel
+    // puts it back in [iC,oC] order.
+    float4v *red = (float4v *)s_raw;
+    constexpr int BLK = MI * NI * kWave;   // float4 per block
+    __syncthreads();
+    if (wave >= 2) {
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int j = 0; j < NI; j++) red[(wave - 2) * BLK + (i * NI + j) * kWave + lane] = acc[i][j];
+    }
+    __syncthreads();
+    if (wave < 2) {
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int j = 0; j < NI; j++) acc[i][j] += red[wave * BLK + (i * NI + j) * kWave + lane];
+    }
+    __syncthreads();
+    if (wave == 1) {
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int j = 0; j < NI; j++) red[(i * NI + j) * kWave + lane] = acc[i][j];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        float4v *part = (float4v *)(a.partial + ((long)slot * gridDim.y + blockIdx.y) * (kWsBlock * kWsBlock));
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int j = 0; j < NI; j++) part[(i * NI + j) * kWave + lane] = acc[i][j] + red[(i * NI + j) * kWave + lane];
+        if (lane == 0 && blockIdx.y == 0) a.flags[slot] = 1;
+    }
+}
+
+// dw[k][ci][co] = sum of the written slots of offset k, in slot order.  A slot holds one
+// 64x64 block per (iC,oC) block pair, each in accumulator order of MI x NI tiles (see
+// wgrad_wave_kernel).  A workgroup covers 32 consecutive co of one ci; its 8 groups of 32
+// threads each add every 8th slot, and the 8 sub-sums are added in a fixed order.
+template <sph_dtype DT>
+__global__ __launch_bounds__(256) void wgrad_slot_reduce_kernel(const float *partial, const int *flags, int slots_per_k,
+                                                                int iC, int oC, int ni_tiles,
+                                                                typename Traits<DT>::elem *dw)
+{
+    __shared__ float s_sum[8][32];
+    const int k = blockIdx.z, ci = blockIdx.y, co = blockIdx.x * 32 + (threadIdx.x & 31), j = threadIdx.x >> 5;
+    const int sbn = (oC + kWsBlock - 1) / kWsBlock, nblk = ((iC + kWsBlock - 1) / kWsBlock) * sbn;
+    const int bi = ci / kWsBlock, bj = co / kWsBlock, li = ci % kWsBlock, lj = co % kWsBlock;
+    // accumulator order inside the block: tile (li/16, lj/16), lane = 16*((li%16)/4) + lj%16, value li%4
+    const int off = (((li >> 4) * ni_tiles + (lj >> 4)) * kWave + (((li & 15) >> 2) << 4) + (lj & 15)) * 4 + (li & 3);
+    const long blk = (long)kWsBlock * kWsBlock;
+    const float *p = partial + ((long)k * slots_per_k * nblk + bi * sbn + bj) * blk + off;
+    const int *f = flags + (long)k * slots_per_k;
+    float s = 0.f;
+    if (co < oC)
+        for (int c = j; c < slots_per_k; c += 8)
+            if (f[c]) s += p[(long)c * nblk * blk];
+    s_sum[j][threadIdx.x & 31] = s;
+    __syncthreads();
+    if (j == 0 && co < oC) {
+        float t = 0.f;
+#pragma unroll
+        for (int q = 0; q < 8; q++) t += s_sum[q][threadIdx.x];
+        dw[((long)k * iC + ci) * oC + co] = (typename Traits<DT>::elem)t;
+    }
+}
+
 inline int elem_size(sph_dtype dt) { return dt == SPH_F32 ? 4 : (dt == SPH_I8 ? 1 : 2); }
 inline int frag_elems(sph_dtype dt) { return 16 / elem_size(dt); }
 inline int pad_waves(int ndim)
@@ -699,19 +1006,70 @@ int launch_pack(const void *w, int KV, int kdim, int ndim, long sk, long skk, lo
     return sph_check_launch("sph_weight_pack");
 }
 
+// 16-channel tiles of one side of the widest block: 1, 2 or 4
+inline int wgrad_tiles(int channels)
+{
+    const int t = sph_div_up(channels < kWsBlock ? channels : kWsBlock, 16);
+    return t <= 1 ? 1 : (t <= 2 ? 2 : 4);
+}
+inline size_t wgrad_wave_lds(int e, int mi, int ni)
+{
+    const int pb = (e == 2 ? 2 : 1) * SPH_GROUP;
+    const size_t stage = (size_t)4 * pb * ((mi * 16 * e + 16) + (ni * 16 * e + 16));
+    const size_t red = (size_t)2 * mi * ni * kWave * 4 * sizeof(float); // two waves' blocks at once
+    return stage > red ? stage : red;
+}
+inline int wgrad_wave_chunks(int ntiles) { return ntiles < 1 ? 1 : sph_div_up(ntiles, kWsTiles); }
+inline bool wgrad_wave_ok(sph_dtype dt, int iC, int oC)
+{
+    const int e = elem_size(dt);
+    return (iC * e) % 16 == 0 && (oC * e) % 16 == 0;
+}
+
 template <sph_dtype DT>
-int launch_wgrad(const WgradArgs &a, void *dw, hipStream_t st)
+int launch_wgrad(const WgradArgs &a0, void *dw, hipStream_t st)
 {
     typedef typename Traits<DT>::elem elem;
+    const int KV = a0.book.KV;
+    const int per_k = a0.iC * a0.oC;
+    const long total = (long)KV * per_k;
+    const bool aligned = ((uintptr_t)a0.feat % 16 == 0) && ((uintptr_t)a0.dout % 16 == 0);
+    const bool small = (double)a0.in_rows * a0.iC * sizeof(elem) < 4294967296.0 &&
+                       (double)a0.out_rows * a0.oC * sizeof(elem) < 4294967296.0 &&
+                       (double)a0.ntiles * a0.cap * SPH_GROUP < 2147483648.0;
+    if (wgrad_wave_ok(DT, a0.iC, a0.oC) && aligned && small && a0.in_rows > 0 && a0.out_rows > 0) {
+        WgradArgs a = a0;
+        const int sb = sph_div_up(a.iC, kWsBlock) * sph_div_up(a.oC, kWsBlock);
+        a.nchunk = wgrad_wave_chunks(a.ntiles);
+        a.nslots = KV * a.nchunk * kWsSlices;
+        a.flags = (int *)(a.partial + (size_t)a.nslots * sb * kWsBlock * kWsBlock);
+        const dim3 grid(sph_xcd_grid(KV * a.nchunk) * kWsSlices, sb);
+        const int mi = wgrad_tiles(a.iC), ni = wgrad_tiles(a.oC);
+        int rc;
+#define SPH_WGRAD_CASE(M, N)                                                                      \
+    if (mi == M && ni == N) {                                                                     \
+        const size_t lds = wgrad_wave_lds((int)sizeof(elem), M, N);                               \
+        rc = set_lds(wgrad_wave_kernel<DT, M, N>, lds);                                           \
+        if (rc) return rc;                                                                        \
+        hipLaunchKernelGGL((wgrad_wave_kernel<DT, M, N>), grid, dim3(256), lds, st, a);           \
+    }
+        SPH_WGRAD_CASE(1, 1) SPH_WGRAD_CASE(1, 2) SPH_WGRAD_CASE(1, 4)
+        SPH_WGRAD_CASE(2, 1) SPH_WGRAD_CASE(2, 2) SPH_WGRAD_CASE(2, 4)
+        SPH_WGRAD_CASE(4, 1) SPH_WGRAD_CASE(4, 2) SPH_WGRAD_CASE(4, 4)
+#undef SPH_WGRAD_CASE
+        rc = sph_check_launch("sph_conv_wgrad");
+        if (rc) return rc;
+        hipLaunchKernelGGL(wgrad_slot_reduce_kernel<DT>, dim3((unsigned)((a.oC + 31) / 32), a.iC, KV), dim3(256), 0, st,
+                           a.partial, a.flags, a.nchunk * kWsSlices, a.iC, a.oC, ni, (elem *)dw);
+        return sph_check_launch("sph_conv_wgrad(reduce)");
+    }
+    const WgradArgs &a = a0;
     constexpr int LDP = 4 * Traits<DT>::KW + 16 / (int)sizeof(elem);
     const int iCp = (a.iC + 15) & ~15, oCp = (a.oC + 15) & ~15;
     size_t lds = (size_t)(iCp + oCp) * LDP * sizeof(elem);
-    const int KV = a.book.KV;
     hipLaunchKernelGGL(wgrad_kernel<DT>, dim3(KV * a.nchunk), dim3(kWgThreads), lds, st, a);
     int rc = sph_check_launch("sph_conv_wgrad");
     if (rc) return rc;
-    int per_k = a.iC * a.oC;
-    long total = (long)KV * per_k;
     hipLaunchKernelGGL(wgrad_reduce_kernel<DT>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
                        a.partial, KV, a.nchunk, per_k, (elem *)dw);
     return sph_check_launch("sph_conv_wgrad(reduce)");
@@ -794,7 +1152,12 @@ SPH_EXPORT int sph_conv_apply(sph_dtype dt, const void *feature, int feature_row
 SPH_EXPORT size_t sph_wgrad_partial_elems(int KV, int iC, int oC, int out_rows)
 {
     if (KV <= 0 || iC <= 0 || oC <= 0) return 0;
-    return (size_t)KV * wgrad_chunks(sph_book_tiles(out_rows)) * iC * oC;
+    const int ntiles = sph_book_tiles(out_rows);
+    const size_t general = (size_t)KV * wgrad_chunks(ntiles) * iC * oC;
+    const size_t slots = (size_t)KV * wgrad_wave_chunks(ntiles) * kWsSlices;
+    const size_t blocks = (size_t)sph_div_up(iC, kWsBlock) * sph_div_up(oC, kWsBlock);
+    const size_t fast = slots * blocks * kWsBlock * kWsBlock + slots; // 64x64 blocks + one flag word per slot
+    return general > fast ? general : fast;
 }
 
 SPH_EXPORT int sph_conv_wgrad(sph_dtype dt, const void *feature, int in_rows, int iC, const void *d_out,
