@@ -469,13 +469,38 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
                 }
             }
         } else {
-            for (int row = lane / cpr; row < nrows; row += rstep) {
-                const uint32_t *src = &s_acc[row * LDW + col0 + ch * VE];
-                union { int4v v; elem e[VE]; } u;
+            // scale / shift of this lane's VE columns stay in registers for all rows
+            float sc[VE], sh[VE];
 #pragma unroll
-                for (int j = 0; j < VE; j++)
-                    u.e[j] = to_elem<DT>(epilogue_value<DT>(a, src[j], col0 + ch * VE + j));
-                *(int4v *)(out + (long)row * a.ndim + ch * VE) = u.v;
+            for (int j = 0; j < VE; j++) {
+                sc[j] = a.scale ? a.scale[col0 + ch * VE + j] : 1.f;
+                sh[j] = (DT != SPH_I8 && a.shift) ? a.shift[col0 + ch * VE + j] : 0.f;
+            }
+            const bool relu = DT != SPH_I8 && a.relu;
+            constexpr int UR = VE > 8 ? 2 : 4;
+            for (int row0 = lane / cpr; row0 < nrows; row0 += UR * rstep) {
+                int4v f[UR][VE / 4];
+#pragma unroll
+                for (int q = 0; q < UR; q++) {
+                    const int row = min(row0 + q * rstep, nrows - 1);
+#pragma unroll
+                    for (int j = 0; j < VE / 4; j++)
+                        f[q][j] = *(const int4v *)&s_acc[row * LDW + col0 + ch * VE + j * 4];
+                }
+#pragma unroll
+                for (int q = 0; q < UR; q++) {
+                    const int row = row0 + q * rstep;
+                    union { int4v v; elem e[VE]; } u;
+#pragma unroll
+                    for (int j = 0; j < VE; j++) {
+                        const int raw = j % 4 == 0 ? f[q][j / 4].x : (j % 4 == 1 ? f[q][j / 4].y : (j % 4 == 2 ? f[q][j / 4].z : f[q][j / 4].w));
+                        float v = DT == SPH_I8 ? (float)raw : __builtin_bit_cast(float, raw);
+                        v = v * sc[j] + sh[j];
+                        if (relu) v = v > 0.f ? v : 0.f;
+                        u.e[j] = to_elem<DT>(v);
+                    }
+                    if (row < nrows) *(int4v *)(out + (long)row * a.ndim + ch * VE) = u.v;
+                }
             }
         }
     } else {
@@ -767,18 +792,21 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
     // so that several batches stay in flight; slots without a pair are zeroed when the rows
     // are staged.  Returns the mask of pairs that exist.
     auto gather = [&](int idx, int4v (&ra)[MI], int4v (&rg)[NI]) -> unsigned {
+        // all lane exchanges first, then all loads: one wait on the LDS queue instead of one per row
         const int other = __shfl_xor(idx, 32, kWave);
+        int rowA[MI], rowG[NI];
+#pragma unroll
+        for (int it = 0; it < MI; it++) rowA[it] = __shfl(idx, pairA[it], kWave);
+#pragma unroll
+        for (int it = 0; it < NI; it++) rowG[it] = __shfl(idx, 32 + pairG[it], kWave);
+        __builtin_amdgcn_sched_barrier(0);
         const unsigned ok = (unsigned)__ballot(idx >= 0 && other >= 0);
 #pragma unroll
-        for (int it = 0; it < MI; it++) {
-            const int row = max(__shfl(idx, pairA[it], kWave), 0);
-            ra[it] = *(const int4v *)(a.feat + ((unsigned)row * strideA + (unsigned)srcA[it]));
-        }
+        for (int it = 0; it < MI; it++)
+            ra[it] = *(const int4v *)(a.feat + ((unsigned)max(rowA[it], 0) * strideA + (unsigned)srcA[it]));
 #pragma unroll
-        for (int it = 0; it < NI; it++) {
-            const int orow = max(__shfl(idx, 32 + pairG[it], kWave), 0);
-            rg[it] = *(const int4v *)(a.dout + ((unsigned)orow * strideG + (unsigned)srcG[it]));
-        }
+        for (int it = 0; it < NI; it++)
+            rg[it] = *(const int4v *)(a.dout + ((unsigned)max(rowG[it], 0) * strideG + (unsigned)srcG[it]));
         return ok;
     };
     auto stage = [&](unsigned ok, const int4v (&ra)[MI], const int4v (&rg)[NI]) {
