@@ -9,10 +9,12 @@
 // atomics, summation order fixed by the book.  conv_apply_kernel is the general
 // fallback for unaligned or very long rows.
 //
-// wgrad (sph_conv_wgrad): a workgroup owns (kernel offset, range of tiles),
-// transposes gathered rows through LDS so that the pair index becomes the MFMA
-// K dimension, keeps the [iC,oC] block in registers and writes one fp32 partial;
-// a second kernel sums the partials in a fixed order.
+// wgrad (sph_conv_wgrad): work items are (kernel offset, chunk of 64 tiles, slice of 64
+// groups); a wave gathers 32 pairs' rows with 16-byte loads into its own LDS area and
+// reads MFMA operands with the pair index as the K dimension through transposing LDS
+// reads; the [64,64] block stays in registers, one fp32 partial per workgroup, summed
+// in a fixed order by a second kernel.  wgrad_kernel is the general fallback for rows
+// that are not whole 16-byte chunks.
 #include "common.h"
 
 namespace {
@@ -631,19 +633,21 @@ __global__ void wgrad_reduce_kernel(const float *partial, int KV, int nchunk, in
 // ---------------------------------------------------------------------------
 // wgrad, fast path (rows are whole 16-byte chunks).
 //
-// Work item = (offset k, chunk of 64 tiles, slice of 64 groups of that chunk's
-// groups at k, 64x64 block of [iC,oC]).  A chunk holds at most 64*8 groups per
-// offset, so 8 slices always cover it; slices beyond the chunk's real group count
-// exit at once (a submanifold book has 8 groups per tile at the centre offset and
-// about one elsewhere: slicing by groups, not tiles, is what balances the grid).
-// The four waves of the workgroup take the slice's batches (2 groups = 32 pairs)
-// round robin and never synchronise until the end: a wave gathers the 32 feature
-// rows and 32 d_out rows with 16-byte loads into its own LDS area in natural
-// [pair][channel] order, and reads MFMA operands with the pair index as the K
-// dimension through transposing LDS reads (16-bit types) or strided 4-byte reads
-// (fp32).  The [64,64] block lives in registers; the workgroup's four blocks are
-// summed through LDS into one fp32 partial, and wgrad_slot_reduce_kernel adds
-// the written slots in a fixed order.
+// Work item = (offset k, chunk of 64 tiles, slice of 64 groups of that chunk's groups at
+// k, 64x64 block of [iC,oC]).  A chunk holds at most 64*8 groups per offset; four
+// workgroups are launched per (offset, chunk), workgroup h takes slices h and h+4, and
+// those whose first slice lies beyond the chunk's real group count exit at once (a
+// submanifold book has 8 groups per tile at the centre offset and about one elsewhere:
+// slicing by groups, not tiles, is what balances the grid).
+// The four waves of the workgroup take the slice's batches (32 pairs; 16 for fp32) round
+// robin and never synchronise until the end: a wave gathers the batch's feature rows and
+// d_out rows with 16-byte loads into its own LDS area in natural [pair][channel] order,
+// and reads MFMA operands with the pair index as the K dimension through transposing
+// LDS reads (16-bit types) or strided 4-byte reads (fp32).  The block lives in registers;
+// the workgroup's four blocks are summed through LDS into one fp32 partial, and
+// wgrad_slot_reduce_kernel adds the written slots in a fixed order.
+// What bounds it (64->64 fp16, 8 waves per CU): LDS traffic (8 KiB staged and 8 KiB read
+// back per batch and wave) and the MFMAs, about equally.
 // ---------------------------------------------------------------------------
 constexpr int kWsTiles = 64;   // tiles per chunk (one lane each)
 constexpr int kWsSlice = 64;   // groups per slice

@@ -216,6 +216,42 @@ def test_half_backward(dtype):
     assert (err <= 1e-3 + 1e-2 * np.abs(dw_ref) + 2e-3 * np.sqrt(n)).all()
 
 
+@pytest.mark.parametrize("dtype,ic,oc", [
+    (torch.float16, 8, 24), (torch.float16, 40, 64), (torch.float16, 16, 32),
+    (torch.bfloat16, 128, 64), (torch.bfloat16, 64, 128), (torch.bfloat16, 96, 48),
+    (torch.float32, 72, 40), (torch.float32, 128, 128), (torch.float32, 4, 12),
+])
+@pytest.mark.parametrize("subm", [True, False])
+def test_wgrad_channel_blocks_and_chunks(dtype, ic, oc, subm):
+    """Weight gradient over more than 64 tiles (several chunks, more than four slices at
+    the centre offset) and over channel counts that need several 64x64 blocks, zero-padded
+    16-channel tiles, or the general kernel (rows that are not whole 16-byte chunks)."""
+    case = _random_case(500 + ic + oc, subm, shape=(16, 64, 24), p=0.3)
+    rng = np.random.default_rng(8)
+    n, m = case["sidx"].shape[0], case["oracle"][0].shape[0]
+    assert max(n, m) > 64 * 128
+    feat = torch.tensor(rng.standard_normal((n, ic)), dtype=torch.float32).to(dtype)
+    g = torch.tensor(rng.standard_normal((m, oc)), dtype=torch.float32).to(dtype)
+    book = case["book"]
+    d_w = ext.rule_conv_d_weight(feat.to(G.DEV), g.to(G.DEV), book, None)
+    assert d_w.dtype == dtype and tuple(d_w.shape) == (27, ic, oc)
+    tri = G.oracle_triples(case["oracle"][2], case["oracle"][3])
+    f64, g64 = feat.double().numpy(), g.double().numpy()
+    ref = np.zeros((27, ic, oc))
+    mag = np.zeros((27, ic, oc))
+    for k in np.unique(tri[:, 0]):
+        s = tri[tri[:, 0] == k]
+        ref[k] = f64[s[:, 1]].T @ g64[s[:, 2]]
+        mag[k] = np.abs(f64[s[:, 1]]).T @ np.abs(g64[s[:, 2]])
+    err = np.abs(d_w.double().cpu().numpy() - ref)
+    # fp32 accumulation of the products (1e-5 of their absolute sum) + one rounding to the storage type
+    eps = {torch.float32: 0.0, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
+    assert (err <= 1e-5 * mag + 2 * eps * np.abs(ref) + 1e-6).all()
+    # run-to-run determinism (fixed summation order)
+    again = ext.rule_conv_d_weight(feat.to(G.DEV), g.to(G.DEV), book, None)
+    assert torch.equal(again, d_w)
+
+
 def test_fused_epilogue_scale_shift_relu():
     case = _random_case(41, True)
     rng = np.random.default_rng(7)
