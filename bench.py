@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0
 # (seed 0), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script scaled by a
 # 256 MiB copy (factors 2.000 / 1.000); commands and raw values: profiles/bench_headline_subm64_f16.md.
 # None for any other workload.
-MEASURED_TRAFFIC_BYTES = {"conv": 9613 * 1024 * 2 + 11924 * 1024, "rules": 761 * 1024 * 2 + 3313 * 1024}
+MEASURED_TRAFFIC_BYTES = {"conv": 9595 * 1024 * 2 + 11924 * 1024, "rules": 761 * 1024 * 2 + 3313 * 1024}
 
 
 def parse():
@@ -35,6 +35,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--backward", action="store_true",
+                    help="also time dgrad (transposed rule book + kernel) and wgrad of the same layer; "
+                         "reported under 'kernels', not part of 'value'")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 256 MiB device-to-device copies (a kernel of known HBM traffic, "
@@ -165,13 +168,21 @@ def main():
     pack_ms = event_ms(lambda: lib.sph_weight_pack(L.F16, w.data_ptr(), 27, ic, oc, ic * oc, oc, 1,
                                                    packed.data_ptr(), stream), iters, torch)
     assert torch.equal(out_buf, out)
+    extra = {}
+    if args.backward:
+        d_out = torch.tensor(rng.standard_normal((n, oc)), dtype=torch.float32, device=dev).half()
+        w_t = w.permute(0, 2, 1).contiguous()
+        extra["transposed_rulegen_ms"] = event_ms(lambda: book._build(True), iters, torch)
+        book.transposed()
+        extra["dgrad_ms"] = event_ms(lambda: ext.rule_conv_d_feature(d_out, w_t, book, None, None, n), iters, torch)
+        extra["wgrad_ms"] = event_ms(lambda: ext.rule_conv_d_weight(feat, d_out, book, None), iters, torch)
     e = 2
     nt = book.fwd.ntiles
     conv_bytes = n * ic * e + n * oc * e + 27 * ic * oc * e + 8 * P
     rule_bytes = 4 * z_ptr.numel() + 4 * n + 8 * P + nt * (4 + 2 * 28)
     conv_flops = 2.0 * P * ic * oc
     if conv_ms >= rulegen_ms:
-        dom = {"kernel": "conv_wave_kernel<f16,2,4>", "bytes": conv_bytes, "ms": conv_ms, "key": "conv"}
+        dom = {"kernel": "conv_wave_kernel<f16,2,4,false>", "bytes": conv_bytes, "ms": conv_ms, "key": "conv"}
     else:
         dom = {"kernel": "build_book_kernel<false>", "bytes": rule_bytes, "ms": rulegen_ms, "key": "rules"}
     achieved = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
@@ -192,7 +203,7 @@ def main():
         "kernels": {"rulegen_ms": rulegen_ms, "weight_pack_ms": pack_ms, "conv_forward_ms": conv_ms,
                     "rulegen_GBps": rule_bytes / (rulegen_ms * 1e-3) / 1e9,
                     "conv_GBps": conv_bytes / (conv_ms * 1e-3) / 1e9,
-                    "conv_TFLOPs": conv_flops / (conv_ms * 1e-3) / 1e12},
+                    "conv_TFLOPs": conv_flops / (conv_ms * 1e-3) / 1e12, **extra},
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:
