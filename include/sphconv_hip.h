@@ -184,6 +184,18 @@ int sph_conv_wgrad(sph_dtype dt, const void *feature, int in_rows, int iC, const
  * reorderFeatureKernel / reorderFeatureBackwardKernel (tensor.cu:39-76,130-145). */
 int sph_permute_rows(const void *src, const int32_t *index, int rows, int row_bytes,
                      int gather, void *out, void *stream);
+/* Replaces init_tensor's index work (src/sphconv/tensor.cu:78-127 with fillGridKernel 21-36
+ * and the index half of reorderFeatureKernel 39-76): COO coordinates `indices` [n,4] int32
+ * (b, s0, s1, s2) -> z_idx [n], z_ptr [B*S0*S1] (inclusive counts) and permutation [n]
+ * (input row r becomes row permutation[r]; move the features with sph_permute_rows,
+ * gather = 0).  Fibers come out in ascending S2 order.  status [2] int32 (device) receives
+ * the number of coordinates outside the grid and the number of duplicated coordinates;
+ * the outputs are only meaningful when both are 0.  `workspace` is device memory of at
+ * least sph_init_tensor_workspace(...) bytes, 256-byte aligned; nothing is allocated. */
+size_t sph_init_tensor_workspace(int n, int B, int S0, int S1, int S2);
+int sph_init_tensor(const int32_t *indices, int n, int B, int S0, int S1, int S2, int32_t *z_idx,
+                    int32_t *z_ptr, int32_t *permutation, int32_t *status, void *workspace,
+                    size_t workspace_bytes, void *stream);
 /* Replaces to_dense / to_dense_backward (tensor.cu:222-309): dense is
  * [B,S0,S1,S2,C]; only active cells are written (forward) / read (backward). */
 int sph_to_dense(const void *feature, const int32_t *z_idx, const int32_t *z_ptr, int rows,

@@ -62,6 +62,8 @@ _SIGNATURES = {
     "sph_conv_apply": (_I, [_I, _P, _I, _I, _P, _I, C.POINTER(Book), C.POINTER(Epilogue), _P, _P]),
     "sph_wgrad_partial_elems": (_Z, [_I, _I, _I, _I]),
     "sph_conv_wgrad": (_I, [_I, _P, _I, _I, _P, _I, C.POINTER(Book), _P, _P, _P]),
+    "sph_init_tensor_workspace": (_Z, [_I, _I, _I, _I, _I]),
+    "sph_init_tensor": (_I, [_P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _Z, _P]),
     "sph_permute_rows": (_I, [_P, _P, _I, _I, _I, _P, _P]),
     "sph_to_dense": (_I, [_P, _P, _P, _I, _I, _I, _I, _P, _P]),
     "sph_to_dense_backward": (_I, [_P, _P, _P, _I, _I, _I, _I, _P, _P]),

@@ -76,7 +76,8 @@ def init_tensor(feature: torch.Tensor, indicesBZYX: torch.Tensor, batchSize: int
                 spatialShape: Sequence[int]) -> List[torch.Tensor]:
     """tensor.cu:78-127 -> [outFeature, zIndices, zPtr, permutation].  Rows of a
     fiber are ordered by ascending S2 (one legal order of the reference's output).
-    Sorting and the prefix sum use torch device ops; the row move is a HIP kernel."""
+    One 8-byte device->host read checks the coordinates (the reference checks nothing:
+    coordinates outside the grid or duplicated ones corrupt its output)."""
     if indicesBZYX.dtype != torch.int32 or indicesBZYX.dim() != 2 or indicesBZYX.shape[1] != 4:
         raise ValueError("indices must be int32 [NNZ,4] (b,s0,s1,s2)")
     if feature.dim() != 2 or feature.shape[0] != indicesBZYX.shape[0]:
@@ -85,24 +86,27 @@ def init_tensor(feature: torch.Tensor, indicesBZYX: torch.Tensor, batchSize: int
     B = int(batchSize)
     n = feature.shape[0]
     dev = feature.device
-    idx = indicesBZYX.long()
-    if n:
-        lim = torch.tensor([B, S0, S1, S2], device=dev)
-        if bool(((idx < 0) | (idx >= lim)).any()):
-            raise ValueError("voxel coordinate outside batch/spatial shape %s" % ([B, S0, S1, S2],))
-    key = ((idx[:, 0] * S0 + idx[:, 1]) * S1 + idx[:, 2]) * S2 + idx[:, 3]
-    skey, order = torch.sort(key)
-    if n > 1 and bool((skey[1:] == skey[:-1]).any()):
-        raise ValueError("duplicate voxel coordinates")
-    z_idx = (skey % S2).to(torch.int32)
-    counts = torch.bincount(torch.div(skey, S2, rounding_mode="floor"), minlength=B * S0 * S1)
-    z_ptr = torch.cumsum(counts, 0).to(torch.int32).view(B, S0, S1)
+    lib = L.lib()
+    idx = indicesBZYX.contiguous()
+    z_idx = torch.empty(n, dtype=torch.int32, device=dev)
+    z_ptr = torch.empty((B, S0, S1), dtype=torch.int32, device=dev)
     permutation = torch.empty(n, dtype=torch.int32, device=dev)
-    permutation[order] = torch.arange(n, dtype=torch.int32, device=dev)
+    status = torch.empty(2, dtype=torch.int32, device=dev)
+    nbytes = lib.sph_init_tensor_workspace(n, B, S0, S1, S2)
+    if nbytes == 0:
+        raise L.SphconvError("bad batch size / spatial shape %s" % ([B, S0, S1, S2],))
+    work = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    L.check(lib.sph_init_tensor(L.ptr(idx), n, B, S0, S1, S2, L.ptr(z_idx), L.ptr(z_ptr), L.ptr(permutation),
+                                L.ptr(status), L.ptr(work), nbytes, L.stream()))
+    outside, dup = (int(v) for v in status.tolist())
+    if outside:
+        raise ValueError("voxel coordinate outside batch/spatial shape %s" % ([B, S0, S1, S2],))
+    if dup:
+        raise ValueError("duplicate voxel coordinates")
     feature = feature.contiguous()
     out = torch.empty_like(feature)
-    L.check(L.lib().sph_permute_rows(L.ptr(feature), L.ptr(permutation), n,
-                                     feature.shape[1] * feature.element_size(), 0, L.ptr(out), L.stream()))
+    L.check(lib.sph_permute_rows(L.ptr(feature), L.ptr(permutation), n,
+                                 feature.shape[1] * feature.element_size(), 0, L.ptr(out), L.stream()))
     return [out, z_idx, z_ptr, permutation]
 
 

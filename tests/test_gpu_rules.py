@@ -186,3 +186,34 @@ def test_extension_functions_match_reference_signatures():
     bad = idx.copy(); bad[0, 3] = 99
     with pytest.raises(ValueError):
         ext.init_tensor(G.t(feat), G.t(bad), 2, [8, 9, 9])
+
+
+@pytest.mark.parametrize("B,shape,n", [(1, (64, 512, 32), 40000), (3, (7, 5, 3), 50), (2, (2048, 2048, 1024), 3000),
+                                       (1, (4, 4, 4), 0), (1, (1, 1, 1), 1)])
+def test_init_tensor_sizes(B, shape, n):
+    """COO -> compressed layout at sizes that need more than 32 key bits, one cell, no voxel
+    at all; checked against the oracle and against the defining invariants."""
+    rng = np.random.default_rng(B * 1000 + n)
+    cells = B * shape[0] * shape[1] * shape[2]
+    lin = np.unique(rng.integers(0, cells, size=n, dtype=np.int64))[:n] if n else np.zeros(0, np.int64)
+    rng.shuffle(lin)
+    idx = np.stack(np.unravel_index(lin, (B,) + tuple(shape)), axis=1).astype(np.int32).reshape(-1, 4)
+    feat = rng.standard_normal((idx.shape[0], 5)).astype(np.float32)
+    f, z_idx, z_ptr, perm = ext.init_tensor(G.t(feat), G.t(idx), B, list(shape))
+    f, z_idx, z_ptr, perm = f.cpu().numpy(), z_idx.cpu().numpy(), z_ptr.cpu().numpy(), perm.cpu().numpy()
+    # invariants: inclusive counts per column, ascending S2 inside a fiber, rows follow the permutation
+    col = (idx[:, 0].astype(np.int64) * shape[0] + idx[:, 1]) * shape[1] + idx[:, 2]
+    counts = np.bincount(col, minlength=B * shape[0] * shape[1])
+    assert np.array_equal(z_ptr.reshape(-1), np.cumsum(counts))
+    assert np.array_equal(np.sort(perm), np.arange(idx.shape[0]))
+    assert np.array_equal(f[perm], feat) and np.array_equal(z_idx[perm], idx[:, 3])
+    order = np.argsort(lin, kind="stable")
+    assert np.array_equal(perm[order], np.arange(idx.shape[0]))
+    if cells < 1 << 24:
+        f2, z2, p2, perm2 = O.init_tensor(feat, idx, B, list(shape))
+        assert np.array_equal(f, f2) and np.array_equal(z_idx, z2) and np.array_equal(z_ptr, p2)
+        assert np.array_equal(perm, perm2)
+    # backward of the row move
+    g = rng.standard_normal(f.shape).astype(np.float32)
+    back = ext.init_tensor_backward(G.t(g), G.t(perm)).cpu().numpy()
+    assert np.array_equal(back, g[perm])
