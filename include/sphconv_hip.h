@@ -204,6 +204,20 @@ int sph_to_dense_backward(const void *d_dense, const int32_t *z_idx, const int32
                           int rows, int ncol, int S2, int row_bytes, void *d_feature,
                           void *stream);
 
+/* Replaces the numpy body of xyz2RangeVoxel (sphconv/data.py:75-128): `points` [m,ndim] float32
+ * on the device (x, y, z first) -> one voxel per pixel of a v_res x h_res range image:
+ * feature [ndim, v_res, h_res] (the winning point's values, 0 elsewhere), depth [v_res, h_res]
+ * (depth bin), thick [v_res, h_res] (1 where a point landed).  Angles in radians:
+ * v0 / h0 = lower bounds of the polar / azimuth range, dtheta / dphi = bin sizes; depth bin =
+ * (log(r) - d0) / dr with d0 = log(d_range[0]) if use_log, else (r - d0) / dr.  Among points
+ * that share a pixel the one with the largest index wins (the reference's "later points
+ * overwrite earlier ones", data.py:106-108).  `winner` is scratch of v_res*h_res int32;
+ * idx_out (optional, [m,3] int32) receives each point's (theta, phi, depth) bins. */
+int sph_xyz_to_rangevoxel(const float *points, int m, int ndim, int v_res, int h_res, int d_res,
+                          float v0_rad, float h0_rad, float dtheta, float dphi, float d0, float dr,
+                          int use_log, int32_t *winner, float *feature, int32_t *depth, int32_t *thick,
+                          int32_t *idx_out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -230,3 +230,54 @@ def rule_conv_i8(feature, weight, scale, rules, rule_size, out_nnz, return_acc=F
     lib().orc_rule_conv_i8(_p(feature), _p(weight), _p(scale), _p(rules), _p(rule_size), ntile,
                            kv, n_max, ic, oc, int(out_nnz), _p(acc), _p(out))
     return (out, acc) if return_acc else out
+
+
+def xyz2rangevoxel(points, v_res=64, h_res=512, d_res=512, v_range=(87.5, 103.4), h_range=(-45, 45),
+                   d_range=(6, 70.4), log=True):
+    """numpy restatement of xyz2RangeVoxel (reference sphconv/data.py:75-128) for float32 points.
+    The reference mixes float32 arrays with float64 numpy scalars; under the promotion rules of
+    the numpy it was written for, each scalar enters the float32 operation rounded to float32 --
+    written out here with explicit float32 casts so that the result does not depend on the numpy
+    version.  Returns (feature [1,C,1,V,H], depth [1,1,V,H] int32, thick [1,V,H] int32,
+    per-point (theta, phi, depth) bins [M,3] int32 and the unclamped float bins [M,3])."""
+    f32 = np.float32
+    pts = np.ascontiguousarray(points, dtype=np.float32)
+    x, y, z = pts[:, 0], pts[:, 1], pts[:, 2]
+    channel = pts.shape[1]
+    with np.errstate(all="ignore"):
+        x2y2 = x * x + y * y                                   # data.py:80
+        r = np.sqrt(x2y2 + z * z)                              # :81
+        thetas = np.arccos(z / r)                              # :82
+        phis = np.arcsin(y / np.sqrt(x2y2))                    # :83
+        delta_phi = f32(np.radians(h_range[1] - h_range[0]) / h_res)      # :85
+        delta_theta = f32(np.radians(v_range[1] - v_range[0]) / v_res)    # :86
+        tf = (thetas - f32(np.radians(v_range[0]))) / delta_theta         # :88
+        pf = (phis - f32(np.radians(h_range[0]))) / delta_phi             # :89
+        if log:
+            delta_r = f32((np.log(d_range[1]) - np.log(d_range[0])) / d_res)   # :92
+            df = (np.log(r) - f32(np.log(d_range[0]))) / delta_r               # :93
+        else:
+            delta_r = f32((d_range[1] - d_range[0]) / d_res)                   # :95
+            df = (r - f32(d_range[0])) / delta_r                               # :96
+    assert tf.dtype == np.float32 and pf.dtype == np.float32 and df.dtype == np.float32
+    raw = np.stack([tf, pf, df], axis=1)
+    # astype(int) truncates toward zero; NaN (a point on the z axis) is taken as 0, which is where
+    # the reference's clamp sends the INT_MIN that an x86 conversion of NaN yields
+    def trunc(a):
+        return np.where(np.isnan(a), 0.0, np.trunc(np.clip(np.nan_to_num(a, nan=0.0), -2.0 ** 40, 2.0 ** 40))).astype(np.int64)
+    theta_idx = np.clip(trunc(tf), 0, v_res - 1)               # :103-106
+    phi_idx = np.clip(trunc(pf), 0, h_res - 1)
+    dfc = np.where(np.isnan(df), f32(0), df)
+    dfc = np.where(dfc < 0, f32(0), dfc)                       # :107 (clamped as a float)
+    dfc = np.where(dfc >= d_res, f32(d_res - 1), dfc)          # :108
+    depth_idx = dfc.astype(np.int32)                           # :121
+    # indexed assignment: the later point of a pixel wins (:114-124)
+    feature = np.zeros((1, channel, 1, v_res, h_res), np.float32)
+    depth = np.zeros((1, 1, v_res, h_res), np.int32)
+    thick = np.zeros((1, v_res, h_res), np.int32)
+    for i in range(pts.shape[0]):
+        feature[0, :, 0, theta_idx[i], phi_idx[i]] = pts[i]
+        depth[0, 0, theta_idx[i], phi_idx[i]] = depth_idx[i]
+        thick[0, theta_idx[i], phi_idx[i]] = 1
+    bins = np.stack([theta_idx, phi_idx, depth_idx], axis=1).astype(np.int32)
+    return feature, depth, thick, bins, raw
