@@ -309,6 +309,69 @@ def test_config1_full_size_fp32():
     np.testing.assert_allclose(out, want, rtol=1e-5, atol=1e-5)
 
 
+def _full_size_case(cfg):
+    from sphconv_amd.rulebook import RuleBook
+    d = make_config(cfg, seed=0)
+    shape, B = d["spatial_shape"], d["batch"]
+    subm = cfg != 3
+    zi, zp = G.t(d["z_idx"]), G.t(d["z_ptr"])
+    if subm:
+        oshape = shape
+        book = RuleBook.build_subm(zi, zp, B, shape, [3, 3, 3])
+        ora = O.get_rules_subm(d["z_idx"], d["z_ptr"], B, shape, shape, [3, 3, 3], [1, 1, 1], [1, 1, 1], n_max=512)
+    else:
+        oshape = H.out_shape_of(shape, [3, 3, 3], [2, 2, 2], [1, 1, 1])
+        book = RuleBook.build(zi, zp, B, shape, oshape, [3, 3, 3], [2, 2, 2], [1, 1, 1])
+        ora = O.get_rules(d["z_idx"], d["z_ptr"], B, shape, oshape, [3, 3, 3], [2, 2, 2], [1, 1, 1], n_max=512)
+    assert ora[4] == 0                                   # no pair dropped by the oracle's padded lists
+    return d, book, ora
+
+
+@pytest.mark.parametrize("cfg,ic,oc", [(2, 32, 32), (3, 32, 64), (5, 64, 64)])
+def test_configs_full_size_fp16(cfg, ic, oc):
+    """BASELINE configurations 2, 3 and 5b at full size: fp16 storage / fp32 accumulate against
+    the C oracle (fp32) on the same fp16-rounded inputs; 5b also dgrad and wgrad."""
+    d, book, (oz_idx, _, rules, rule_size, _) = _full_size_case(cfg)
+    rng = np.random.default_rng(cfg)
+    n, m = d["z_idx"].shape[0], oz_idx.shape[0]
+    feat = torch.tensor(rng.standard_normal((n, ic)), dtype=torch.float32).half()
+    w = torch.tensor(_weights(rng, 27, ic, oc)).half()
+    out = ext.rule_conv(feat.to(G.DEV), w.to(G.DEV), book, None, m)
+    assert out.dtype == torch.float16 and tuple(out.shape) == (m, oc)
+    want = O.rule_conv(feat.float().numpy(), w.float().numpy(), rules, rule_size, m)
+    got = out.float().cpu().numpy()
+    # one rounding to fp16 of an fp32 sum of at most 27*ic products (tolerance of north_star: 1e-2 relative)
+    assert (np.abs(got - want) <= 2.0 ** -10 * np.abs(want) + 1e-3).all()
+    if cfg != 5:
+        return
+    g = torch.tensor(rng.standard_normal((m, oc)), dtype=torch.float32).half()
+    w_perm = w.permute(0, 2, 1).contiguous()
+    d_feat, d_w = ext.rule_conv_backward(g.to(G.DEV), feat.to(G.DEV), w_perm.to(G.DEV), book, None, [1, 1])
+    tgs = [-(-d["spatial_shape"][0] // 2), -(-d["spatial_shape"][1] // 2)]
+    df_o, dw_o = O.rule_conv_backward(g.float().numpy(), feat.float().numpy(), w_perm.float().numpy(), rules,
+                                      rule_size, tgs)
+    assert (np.abs(d_feat.float().cpu().numpy() - df_o) <= 2.0 ** -10 * np.abs(df_o) + 1e-3).all()
+    # d_weight sums ~23 000 products per entry (centre offset: 314 000): fp32 association differs
+    # between the oracle and the GPU, both stay within 1e-5 of the sum of absolute products
+    # (E|x||y| = 2/pi for unit normals), plus the rounding to fp16
+    bound = 1e-5 * (2 / np.pi) * rule_size.sum(0)[:, None, None] + 2.0 ** -10 * np.abs(dw_o) + 1e-3
+    assert (np.abs(d_w.float().cpu().numpy() - dw_o) <= 2 * bound).all()
+
+
+def test_config5a_full_size_int8_exact():
+    """BASELINE configuration 5a at full size: int8 x int8 -> int32 -> requantised int8, bit-exact."""
+    d, book, (oz_idx, _, rules, rule_size, _) = _full_size_case(5)
+    rng = np.random.default_rng(55)
+    n = d["z_idx"].shape[0]
+    f8 = rng.integers(-128, 128, (n, 64), dtype=np.int8)
+    w8 = rng.integers(-128, 128, (27, 64, 64), dtype=np.int8)
+    scale = ((rng.random(64) + 0.5) / 3000.0).astype(np.float32)
+    want = O.rule_conv_i8(f8, w8, scale, rules, rule_size, n)
+    got = ext.rule_conv_int8(G.t(f8), G.t(w8), G.t(scale), book, None, n).cpu().numpy()
+    assert np.array_equal(got, want)
+    assert (want == 127).any() and (want == -128).any() and (np.abs(want) < 100).mean() > 0.3
+
+
 def test_errors_are_reported_not_fatal():
     from sphconv_amd import SphconvError
     case = _random_case(51, True)
