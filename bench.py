@@ -2,7 +2,9 @@
 """Benchmark of the sparse-convolution hot path on one MI355X.
 
 One step = rule generation + forward of one 3x3x3 submanifold convolution
-64->64, fp16 storage / fp32 accumulate, on one synthetic LiDAR-like scan
+64->64, fp16 storage / fp32 accumulate (two kernel launches: the rule kernel, which
+also carries the per-step weight packing as extra workgroups, and the convolution),
+on one synthetic LiDAR-like scan
 (config-2 generator: 64 x 2048 x 64 range grid, ~95-120k active voxels), with
 the scan's index arrays, features and weights already resident in HBM.
 
@@ -134,8 +136,10 @@ def main():
         del src, dst
 
     def step():
-        book = RuleBook.build_subm(z_idx, z_ptr, B, shape, [3, 3, 3])
-        return book, ext.rule_conv(feat, w, book, None, n)
+        # rule generation (the weight is put in MFMA fragment order by extra workgroups of the
+        # same launch, every step) + forward
+        book, packed = RuleBook.build_subm(z_idx, z_ptr, B, shape, [3, 3, 3], weight=w)
+        return book, ext.rule_conv(feat, w, book, None, n, packed=packed)
 
     for _ in range(args.warmup):
         step()

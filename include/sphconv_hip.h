@@ -109,6 +109,15 @@ int sph_num_tiles(const sph_geom *g, int T0, int T1);
 int sph_rules_build(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
                     const int32_t *oz_idx, const int32_t *oz_ptr, int out_rows,
                     const sph_geom *g, int transposed, const sph_book *book, void *stream);
+/* sph_rules_build with a weight pack (sph_weight_pack, same arguments) riding along as extra
+ * workgroups of the same launch: for a layer whose rules are not cached yet, the forward pass
+ * then is two launches (rules + pack, convolution) instead of three.  No reference counterpart
+ * beyond get_rules* (rules.cu:326-486) and the weight argument of rule_conv (rule_conv.cu:286). */
+int sph_rules_build_pack(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
+                         const int32_t *oz_idx, const int32_t *oz_ptr, int out_rows,
+                         const sph_geom *g, int transposed, const sph_book *book,
+                         sph_dtype dt, const void *w, int KV, int kdim, int ndim, long stride_k,
+                         long stride_kk, long stride_n, void *packed, void *stream);
 
 /* Replaces the output-coordinate half of get_rules (rules.cu:417-443, 461-462),
  * in two steps because the caller must size oz_idx:

@@ -87,23 +87,29 @@ class Conv3d(Convolution):
                          _triple(padding), _triple(dilation), groups, tile_size, bias, subm, name,
                          indice_key=indice_key, **kwargs)
 
-    def _rules(self, input: SparseConvTensor, out_shape):
+    def _rules(self, input: SparseConvTensor, out_shape, weight=None):
         """Rule book of this layer on ``input``, shared through ``rule_cache`` when an
-        ``indice_key`` is set (conv.py:159-177)."""
+        ``indice_key`` is set (conv.py:159-177).  Returns the cache entry and, when the
+        rules had to be generated, the weight packed by the same launch (else None)."""
         cached = input.find_rule(self.indice_key)
         if cached is not None:
-            return cached
+            return cached, None
         in_shape = [input.D, input.W, input.H]
+        if weight is not None and weight.dtype != input.feature.dtype:
+            weight = None
         if self.subm:
             book = RuleBook.build_subm(input.z_idx, input.z_ptr, input.B, in_shape, self.kernel_size,
-                                       self.padding, self.dilation)
+                                       self.padding, self.dilation, weight=weight)
         else:
             book = RuleBook.build(input.z_idx, input.z_ptr, input.B, in_shape, out_shape,
-                                  self.kernel_size, self.stride, self.padding, self.dilation)
+                                  self.kernel_size, self.stride, self.padding, self.dilation, weight=weight)
+        packed = None
+        if weight is not None:
+            book, packed = book
         entry = (book.oz_idx, book.oz_ptr, book, None, get_tile_grid_shape(out_shape, self.tile_size))
         if self.indice_key is not None:
             input.rule_cache[self.indice_key] = entry
-        return entry
+        return entry, packed
 
     def forward(self, input: SparseConvTensor) -> SparseConvTensor:
         assert self.in_channels == input.C, \
@@ -111,11 +117,11 @@ class Conv3d(Convolution):
         in_shape = [input.D, input.W, input.H]
         out_shape = in_shape if self.subm else out_spatial(in_shape, self.kernel_size, self.stride,
                                                             self.padding, self.dilation)
-        oz_idx, oz_ptr, book, rule_size, tile_grid_shape = self._rules(input, out_shape)
-        self.rule_book = book if isinstance(book, RuleBook) else None
         weight = self.weight.view(-1, self.in_channels, self.out_channels)
+        (oz_idx, oz_ptr, book, rule_size, tile_grid_shape), packed = self._rules(input, out_shape, weight)
+        self.rule_book = book if isinstance(book, RuleBook) else None
         out_feature = ConvFunction.apply(input.feature, weight, book, rule_size, tile_grid_shape,
-                                         oz_idx.shape[0])
+                                         oz_idx.shape[0], packed)
         out = SparseConvTensor(out_feature, out_shape, input.B, z_ptr=oz_ptr, z_idx=oz_idx)
         out.rule_cache = input.rule_cache
         return out

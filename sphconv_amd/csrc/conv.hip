@@ -16,6 +16,7 @@
 // in a fixed order by a second kernel.  wgrad_kernel is the general fallback for rows
 // that are not whole 16-byte chunks.
 #include "common.h"
+#include "pack.h"
 
 namespace {
 
@@ -82,30 +83,11 @@ __device__ __forceinline__ int4v mfma_step<SPH_I8>(int4v a, int4v b, int4v d)
 }
 
 // ---------------------------------------------------------------------------
-// Weight packing: packed[k][step][ntile][lane][KW] with
-//   kk = step*4*KW + KW*(lane/16) + j,  n = ntile*16 + lane%16,  zero padded.
+// Weight packing (layout and element copy: pack.h)
 // ---------------------------------------------------------------------------
-template <sph_dtype DT>
-__global__ void pack_weight_kernel(const typename Traits<DT>::elem *w, int KV, int kdim, int ndim, long sk,
-                                   long skk, long sn, int nsteps, int ntn, typename Traits<DT>::elem *packed)
+__global__ void pack_weight_kernel(SphPackJob p)
 {
-    constexpr int KW = Traits<DT>::KW;
-    long total = (long)KV * nsteps * ntn * kWave * KW;
-    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= total) return;
-    int j = (int)(i % KW);
-    long t = i / KW;
-    int lane = (int)(t % kWave);
-    t /= kWave;
-    int nt = (int)(t % ntn);
-    t /= ntn;
-    int st = (int)(t % nsteps);
-    int k = (int)(t / nsteps);
-    int kk = st * 4 * KW + KW * (lane >> 4) + j;
-    int n = nt * 16 + (lane & 15);
-    typename Traits<DT>::elem v = (typename Traits<DT>::elem)0;
-    if (kk < kdim && n < ndim) v = w[k * sk + kk * skk + n * sn];
-    packed[i] = v;
+    sph_pack_element(p, (long)blockIdx.x * blockDim.x + threadIdx.x);
 }
 
 struct ConvArgs {
@@ -940,14 +922,10 @@ __global__ __launch_bounds__(256) void wgrad_slot_reduce_kernel(const float *par
     }
 }
 
-inline int elem_size(sph_dtype dt) { return dt == SPH_F32 ? 4 : (dt == SPH_I8 ? 1 : 2); }
-inline int frag_elems(sph_dtype dt) { return 16 / elem_size(dt); }
-inline int pad_waves(int ndim)
-{
-    int nt = sph_div_up(ndim, 16);
-    return nt <= 1 ? 1 : (nt <= 2 ? 2 : (nt <= 4 ? 4 : 8));
-}
-inline int num_steps(sph_dtype dt, int kdim) { return sph_div_up(kdim, 4 * frag_elems(dt)); }
+inline int elem_size(sph_dtype dt) { return sph_elem_size(dt); }
+inline int frag_elems(sph_dtype dt) { return sph_frag_elems(dt); }
+inline int pad_waves(int ndim) { return sph_pad_waves(ndim); }
+inline int num_steps(sph_dtype dt, int kdim) { return sph_num_steps(dt, kdim); }
 inline int wgrad_chunks(int ntiles) { return ntiles < 32 ? (ntiles < 1 ? 1 : ntiles) : 32; }
 
 template <typename K>
@@ -1025,17 +1003,6 @@ int launch_conv_nw(const ConvArgs &a, int nw, int ntiles, hipStream_t st)
     case 4: return launch_conv<DT, 4>(a, ntiles, st);
     default: return launch_conv<DT, 8>(a, ntiles, st);
     }
-}
-
-template <sph_dtype DT>
-int launch_pack(const void *w, int KV, int kdim, int ndim, long sk, long skk, long sn, void *packed, hipStream_t st)
-{
-    typedef typename Traits<DT>::elem elem;
-    int nsteps = num_steps(DT, kdim), ntn = pad_waves(ndim);
-    long total = (long)KV * nsteps * ntn * kWave * Traits<DT>::KW;
-    hipLaunchKernelGGL(pack_weight_kernel<DT>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                       (const elem *)w, KV, kdim, ndim, sk, skk, sn, nsteps, ntn, (elem *)packed);
-    return sph_check_launch("sph_weight_pack");
 }
 
 // 16-channel tiles of one side of the widest block: 1, 2 or 4
@@ -1124,20 +1091,11 @@ SPH_EXPORT size_t sph_weight_packed_bytes(sph_dtype dt, int KV, int kdim, int nd
 SPH_EXPORT int sph_weight_pack(sph_dtype dt, const void *w, int KV, int kdim, int ndim, long stride_k,
                                long stride_kk, long stride_n, void *packed, void *stream)
 {
-    SPH_REQUIRE(w && packed, SPH_ERR_ARG, "sph_weight_pack: null pointer");
-    SPH_REQUIRE(KV > 0 && KV <= SPH_MAX_KV, SPH_ERR_UNSUPPORTED, "sph_weight_pack: kernel volume %d not in 1..%d", KV, SPH_MAX_KV);
-    SPH_REQUIRE(kdim > 0 && kdim <= SPH_MAX_CHANNELS, SPH_ERR_UNSUPPORTED,
-                "sph_weight_pack: %d input channels not in 1..%d", kdim, SPH_MAX_CHANNELS);
-    SPH_REQUIRE(ndim > 0 && ndim <= 128, SPH_ERR_UNSUPPORTED, "sph_weight_pack: %d output channels not in 1..128", ndim);
-    hipStream_t st = (hipStream_t)stream;
-    switch (dt) {
-    case SPH_F32: return launch_pack<SPH_F32>(w, KV, kdim, ndim, stride_k, stride_kk, stride_n, packed, st);
-    case SPH_F16: return launch_pack<SPH_F16>(w, KV, kdim, ndim, stride_k, stride_kk, stride_n, packed, st);
-    case SPH_BF16: return launch_pack<SPH_BF16>(w, KV, kdim, ndim, stride_k, stride_kk, stride_n, packed, st);
-    case SPH_I8: return launch_pack<SPH_I8>(w, KV, kdim, ndim, stride_k, stride_kk, stride_n, packed, st);
-    }
-    sph_set_error("sph_weight_pack: unknown dtype %d", (int)dt);
-    return SPH_ERR_ARG;
+    int rc = sph_pack_args_ok("sph_weight_pack", dt, w, packed, KV, kdim, ndim);
+    if (rc) return rc;
+    const SphPackJob p = sph_pack_job(dt, w, KV, kdim, ndim, stride_k, stride_kk, stride_n, packed);
+    hipLaunchKernelGGL(pack_weight_kernel, dim3((unsigned)((p.total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, p);
+    return sph_check_launch("sph_weight_pack");
 }
 
 SPH_EXPORT int sph_conv_apply(sph_dtype dt, const void *feature, int feature_rows, int kdim,

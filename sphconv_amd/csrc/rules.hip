@@ -4,6 +4,7 @@
 // atomic counters (src/sphconv/rules.cu) by fiber joins, wave ballots and
 // prefix popcounts.  All kernels are integer and HBM/latency bound.
 #include "common.h"
+#include "pack.h"
 
 namespace {
 
@@ -194,6 +195,9 @@ struct BuildArgs {
     ConvParams cv;
     int cap;
     sph_book book;
+    // optional passenger: workgroups behind the tile workgroups pack a weight (total == 0: none)
+    SphPackJob pack;
+    int tile_blocks;
 };
 
 constexpr int kJoinItems = 5; // (row, k0, k1) items a thread joins per pass, all loads of a pass in flight together
@@ -208,6 +212,12 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     __shared__ int s_tmp, s_flag;
 
     const int tid = threadIdx.x;
+    if ((int)blockIdx.x >= a.tile_blocks) {
+        // a weight rides along with the rule generation: the copy needs a launch of its own
+        // otherwise, which costs more than the copy
+        sph_pack_element(a.pack, (long)(blockIdx.x - a.tile_blocks) * kThreads + tid);
+        return;
+    }
     const int tile = sph_xcd_tile(blockIdx.x, (a.q_rows + R - 1) / R);
     const int KV = a.cv.K0 * a.cv.K1 * a.cv.K2;
     const int K01 = a.cv.K0 * a.cv.K1;
@@ -605,19 +615,18 @@ SPH_EXPORT int sph_num_tiles(const sph_geom *g, int T0, int T1)
     return sph_div_up(g->O[0], T0) * sph_div_up(g->O[1], T1);
 }
 
-SPH_EXPORT int sph_rules_build(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
-                               const int32_t *oz_idx, const int32_t *oz_ptr, int out_rows,
-                               const sph_geom *g, int transposed, const sph_book *book, void *stream)
+static int rules_build(const char *who, const int32_t *z_idx, const int32_t *z_ptr, int in_rows, const int32_t *oz_idx,
+                       const int32_t *oz_ptr, int out_rows, const sph_geom *g, int transposed, const sph_book *book,
+                       const SphPackJob *pack, void *stream)
 {
-    SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_rules_build: bad geometry (kernel volume <= %d)", SPH_MAX_KV);
-    SPH_REQUIRE(book_ok(book), SPH_ERR_ARG, "sph_rules_build: bad book");
-    SPH_REQUIRE(z_ptr && oz_ptr && in_rows >= 0 && out_rows >= 0, SPH_ERR_ARG, "sph_rules_build: bad argument");
-    SPH_REQUIRE((in_rows == 0 || z_idx) && (out_rows == 0 || oz_idx), SPH_ERR_ARG, "sph_rules_build: null index array");
+    SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "%s: bad geometry (kernel volume <= %d)", who, SPH_MAX_KV);
+    SPH_REQUIRE(book_ok(book), SPH_ERR_ARG, "%s: bad book", who);
+    SPH_REQUIRE(z_ptr && oz_ptr && in_rows >= 0 && out_rows >= 0, SPH_ERR_ARG, "%s: bad argument", who);
+    SPH_REQUIRE((in_rows == 0 || z_idx) && (out_rows == 0 || oz_idx), SPH_ERR_ARG, "%s: null index array", who);
     const int KV = g->K[0] * g->K[1] * g->K[2];
-    SPH_REQUIRE(book->KV == KV, SPH_ERR_ARG, "sph_rules_build: book.KV %d != kernel volume %d", book->KV, KV);
+    SPH_REQUIRE(book->KV == KV, SPH_ERR_ARG, "%s: book.KV %d != kernel volume %d", who, book->KV, KV);
     SPH_REQUIRE(book->rows == (transposed ? in_rows : out_rows), SPH_ERR_ARG,
-                "sph_rules_build: book.rows %d does not match the stationary side", book->rows);
-    if (book->rows == 0) return SPH_OK;
+                "%s: book.rows %d does not match the stationary side", who, book->rows);
 
     BuildArgs a;
     Grid3 S{g->S[0], g->S[1], g->S[2]}, O{g->O[0], g->O[1], g->O[2]};
@@ -633,13 +642,43 @@ SPH_EXPORT int sph_rules_build(const int32_t *z_idx, const int32_t *z_ptr, int i
     a.cap = sph_book_cap(KV);
     a.book = *book;
     const int nt = sph_book_tiles(book->rows);
+    a.tile_blocks = book->rows > 0 ? sph_xcd_grid(nt) : 0;
+    int pack_blocks = 0;
+    if (pack) {
+        a.pack = *pack;
+        pack_blocks = (int)((pack->total + kThreads - 1) / kThreads);
+    } else {
+        a.pack.total = 0;
+    }
+    if (a.tile_blocks + pack_blocks == 0) return SPH_OK;
     const size_t lds = (size_t)R * KV * sizeof(int32_t);
     hipStream_t st = (hipStream_t)stream;
     if (!transposed)
-        hipLaunchKernelGGL(build_book_kernel<false>, dim3(sph_xcd_grid(nt)), dim3(kThreads), lds, st, a);
+        hipLaunchKernelGGL(build_book_kernel<false>, dim3(a.tile_blocks + pack_blocks), dim3(kThreads), lds, st, a);
     else
-        hipLaunchKernelGGL(build_book_kernel<true>, dim3(sph_xcd_grid(nt)), dim3(kThreads), lds, st, a);
-    return sph_check_launch("sph_rules_build");
+        hipLaunchKernelGGL(build_book_kernel<true>, dim3(a.tile_blocks + pack_blocks), dim3(kThreads), lds, st, a);
+    return sph_check_launch(who);
+}
+
+SPH_EXPORT int sph_rules_build(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
+                               const int32_t *oz_idx, const int32_t *oz_ptr, int out_rows,
+                               const sph_geom *g, int transposed, const sph_book *book, void *stream)
+{
+    return rules_build("sph_rules_build", z_idx, z_ptr, in_rows, oz_idx, oz_ptr, out_rows, g, transposed, book, nullptr,
+                       stream);
+}
+
+SPH_EXPORT int sph_rules_build_pack(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
+                                    const int32_t *oz_idx, const int32_t *oz_ptr, int out_rows,
+                                    const sph_geom *g, int transposed, const sph_book *book,
+                                    sph_dtype dt, const void *w, int KV, int kdim, int ndim, long stride_k,
+                                    long stride_kk, long stride_n, void *packed, void *stream)
+{
+    int rc = sph_pack_args_ok("sph_rules_build_pack", dt, w, packed, KV, kdim, ndim);
+    if (rc) return rc;
+    const SphPackJob p = sph_pack_job(dt, w, KV, kdim, ndim, stride_k, stride_kk, stride_n, packed);
+    return rules_build("sph_rules_build_pack", z_idx, z_ptr, in_rows, oz_idx, oz_ptr, out_rows, g, transposed, book, &p,
+                       stream);
 }
 
 SPH_EXPORT int sph_outcoords_blocks(const sph_geom *g)

@@ -14,13 +14,15 @@ class ConvFunction(torch.autograd.Function):
     padded tensor together with ``rule_size``."""
 
     @staticmethod
-    def forward(ctx, feature, weight, rules, rule_size, tile_grid_shape: List[int], outNNZ: int):
+    def forward(ctx, feature, weight, rules, rule_size, tile_grid_shape: List[int], outNNZ: int, packed=None):
         book = rules if isinstance(rules, RuleBook) else RuleBook.from_padded(
             rules, rule_size, feature.shape[0], int(outNNZ))
         ctx.save_for_backward(feature, weight)
         ctx.book = book
         ctx.tile_grid_shape = tile_grid_shape
-        return ext.rule_conv(feature, weight, book, None, outNNZ)
+        if packed is not None and weight.dtype != feature.dtype:
+            packed = None                       # packed in the weight's type, the kernel needs the feature's
+        return ext.rule_conv(feature, weight, book, None, outNNZ, packed=packed)
 
     @staticmethod
     def backward(ctx, d_featureOut):
@@ -37,7 +39,7 @@ class ConvFunction(torch.autograd.Function):
             d_feature = ext._apply(d_out, packed, w.shape[2], w.shape[1], book.transposed())
         if ctx.needs_input_grad[1]:
             d_weight = ext.rule_conv_d_weight(feature, d_out, book, None).to(weight.dtype)
-        return d_feature, d_weight, None, None, None, None
+        return d_feature, d_weight, None, None, None, None, None
 
 
 class ToDenseFunction(torch.autograd.Function):

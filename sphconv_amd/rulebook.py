@@ -95,31 +95,61 @@ class RuleBook:
         return L.make_geom(self.batch, self.in_shape, self.out_shape, self.kernel, self.stride,
                            self.padding, self.dilation)
 
-    def _build(self, transposed: bool) -> _Buffers:
+    def _build(self, transposed: bool, weight=None, weight_transposed: bool = False):
+        """Launches the rule kernel.  With ``weight`` [KV,a,b] its fragment-ordered copy (what
+        ``sph_weight_pack`` makes, for the contraction over ``a``, or over ``b`` when
+        ``weight_transposed``) is produced by the same launch and returned with the buffers."""
         rows = self.in_rows if transposed else self.out_rows
         buf = _Buffers(rows, self.kv, self.z_ptr.device)
         g, b = self.geom(), buf.struct()
-        rc = L.lib().sph_rules_build(self.z_idx.data_ptr(), self.z_ptr.data_ptr(), self.in_rows,
+        lib = L.lib()
+        if weight is None:
+            rc = lib.sph_rules_build(self.z_idx.data_ptr(), self.z_ptr.data_ptr(), self.in_rows,
                                      self.oz_idx.data_ptr(), self.oz_ptr.data_ptr(), self.out_rows,
                                      C.byref(g), int(transposed), C.byref(b), L.stream())
+            if rc:
+                L.check(rc)
+            return buf
+        w = weight.detach()
+        if not w.is_contiguous():
+            w = w.contiguous()
+        if not w.is_cuda or w.dim() != 3:
+            raise L.SphconvError("weight must be a GPU tensor [KV,iC,oC]")
+        kv, wa, wb = w.shape
+        kdim, ndim = (wb, wa) if weight_transposed else (wa, wb)
+        skk, sn = (1, wb) if weight_transposed else (wb, 1)
+        dt = L.dtype_code(w.dtype)
+        nbytes = lib.sph_weight_packed_bytes(dt, kv, kdim, ndim)
+        if nbytes == 0:
+            raise L.SphconvError("cannot pack weight of shape %s" % (tuple(w.shape),))
+        packed = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+        rc = lib.sph_rules_build_pack(self.z_idx.data_ptr(), self.z_ptr.data_ptr(), self.in_rows,
+                                      self.oz_idx.data_ptr(), self.oz_ptr.data_ptr(), self.out_rows,
+                                      C.byref(g), int(transposed), C.byref(b), dt, w.data_ptr(), kv, kdim, ndim,
+                                      wa * wb, skk, sn, packed.data_ptr(), L.stream())
         if rc:
             L.check(rc)
-        return buf
+        return buf, packed
 
     @classmethod
     def build_subm(cls, z_idx, z_ptr, batch, shape, kernel, padding=None,
-                   dilation=(1, 1, 1)) -> "RuleBook":
+                   dilation=(1, 1, 1), weight=None):
         """Submanifold rules (replaces get_rules_subm, rules.cu:326-390): stride 1,
-        outputs are the inputs; ``padding`` defaults to K//2 (conv.py:210)."""
+        outputs are the inputs; ``padding`` defaults to K//2 (conv.py:210).
+        With ``weight`` [KV,iC,oC] returns ``(book, packed_weight)``: the layer's weight is
+        put in fragment order by the same kernel launch (pass it to ``rule_conv(..., packed=)``)."""
         _check_index_tensors(z_idx, z_ptr, batch, shape)
         pad = [int(k) // 2 for k in kernel] if padding is None else [int(v) for v in padding]
         rb = cls(z_idx, z_ptr, z_idx, z_ptr, batch, shape, shape, kernel, (1, 1, 1), pad, dilation, True)
-        rb.fwd = rb._build(False)
-        return rb
+        if weight is None:
+            rb.fwd = rb._build(False)
+            return rb
+        rb.fwd, packed = rb._build(False, weight)
+        return rb, packed
 
     @classmethod
     def build(cls, z_idx, z_ptr, batch, in_shape, out_shape, kernel, stride, padding,
-              dilation=(1, 1, 1)) -> "RuleBook":
+              dilation=(1, 1, 1), weight=None):
         """Strided rules (replaces get_rules, rules.cu:405-486): output coordinates
         (oz_ptr inclusive scan, oz_idx ascending per column) and pairs.  One
         device->host read of the output row count, as in the reference (rules.cu:461)."""
@@ -144,8 +174,11 @@ class RuleBook:
                                        L.ptr(oz_ptr), L.ptr(oz_idx), out_rows, L.stream()))
         rb = cls(z_idx, z_ptr, oz_idx, oz_ptr, batch, in_shape, out_shape, kernel, stride, padding,
                  dilation, False)
-        rb.fwd = rb._build(False)
-        return rb
+        if weight is None:
+            rb.fwd = rb._build(False)
+            return rb
+        rb.fwd, packed = rb._build(False, weight)    # (book, packed weight) as in build_subm
+        return rb, packed
 
     @classmethod
     def from_padded(cls, rules, rule_size, in_rows: int, out_rows: int) -> "RuleBook":

@@ -195,16 +195,23 @@ def _check_conv_args(feature, weight):
 
 def rule_conv(feature: torch.Tensor, weight: torch.Tensor, rules, ruleSize, outNNZ: int,
               scale: Optional[torch.Tensor] = None, shift: Optional[torch.Tensor] = None,
-              relu: bool = False) -> torch.Tensor:
+              relu: bool = False, packed: Optional[torch.Tensor] = None) -> torch.Tensor:
     """rule_conv.cu:286-336: out[j] = sum over pairs (k,i,j) feature[i] @ weight[k].
     ``scale``/``shift`` (fp32 [oC]) and ``relu`` fuse y = relu(acc*scale + shift)
-    into the store (no reference counterpart; default off)."""
+    into the store (no reference counterpart; default off).  ``packed``: the
+    fragment-ordered copy of this very ``weight`` that ``RuleBook.build*(..., weight=)``
+    returned, which saves the packing launch."""
     weight = _check_conv_args(feature, weight)
     book = _as_book(rules, ruleSize, feature.shape[0], int(outNNZ))
     if book.out_rows != int(outNNZ) or book.kv != weight.shape[0]:
         raise L.SphconvError("rules hold %d output rows / %d offsets, call says %d / %d"
                              % (book.out_rows, book.kv, int(outNNZ), weight.shape[0]))
-    packed = _packed_weight(weight, False)
+    if packed is None:
+        packed = _packed_weight(weight, False)
+    elif packed.numel() != L.lib().sph_weight_packed_bytes(L.dtype_code(weight.dtype), weight.shape[0],
+                                                           weight.shape[1], weight.shape[2]):
+        raise L.SphconvError("packed weight of %d bytes does not belong to a weight of shape %s"
+                             % (packed.numel(), tuple(weight.shape)))
     return _apply(feature, packed, weight.shape[1], weight.shape[2], book.fwd, scale, shift, relu)
 
 

@@ -12,6 +12,7 @@ import torch
 import helpers as H
 import gpu_helpers as G
 from oracle import oracle as O
+import sphconv_amd
 from sphconv_amd import sphconv_cuda as ext
 from sphconv_amd.synth import make_config
 
@@ -386,3 +387,35 @@ def test_errors_are_reported_not_fatal():
                       torch.zeros((27, 8, 8), device=G.DEV, dtype=torch.float64), book, None, n)
     with pytest.raises(SphconvError):
         ext.rule_conv(torch.zeros((n, 8)), torch.zeros((27, 8, 8)), book, None, n)   # CPU tensors
+
+
+@pytest.mark.parametrize("dtype,ic,oc", [(torch.float16, 64, 64), (torch.float32, 5, 33), (torch.int8, 32, 16),
+                                         (torch.bfloat16, 128, 96)])
+@pytest.mark.parametrize("subm", [True, False])
+def test_weight_packed_by_the_rule_launch(dtype, ic, oc, subm):
+    """The weight copy made by extra workgroups of the rule kernel launch equals sph_weight_pack's,
+    the book equals the one built alone, and rule_conv(packed=) gives the same output bits."""
+    from sphconv_amd.rulebook import RuleBook
+    case = _random_case(900 + ic, subm)
+    rng = np.random.default_rng(9)
+    if dtype == torch.int8:
+        w = torch.tensor(rng.integers(-128, 128, (27, ic, oc)), dtype=torch.int8)
+    else:
+        w = torch.tensor(_weights(rng, 27, ic, oc)).to(dtype)
+    w = w.to(G.DEV)
+    zi, zp = G.t(case["z_idx"]), G.t(case["z_ptr"])
+    if subm:
+        book, packed = RuleBook.build_subm(zi, zp, case["B"], case["shape"], case["kernel"], weight=w)
+    else:
+        book, packed = RuleBook.build(zi, zp, case["B"], case["shape"], case["oshape"], case["kernel"],
+                                      case["stride"], case["padding"], weight=w)
+    assert torch.equal(packed, ext._packed_weight(w, False))
+    assert np.array_equal(G.book_triples(book.fwd), G.book_triples(case["book"].fwd))
+    if dtype == torch.int8:
+        return
+    feat = torch.tensor(rng.standard_normal((zi.shape[0], ic)), dtype=torch.float32).to(dtype).to(G.DEV)
+    a = ext.rule_conv(feat, w, book, None, book.out_rows, packed=packed)
+    b = ext.rule_conv(feat, w, case["book"], None, book.out_rows)
+    assert torch.equal(a, b)
+    with pytest.raises(sphconv_amd.SphconvError):
+        ext.rule_conv(feat, w, book, None, book.out_rows, packed=packed[:-1024])
