@@ -227,6 +227,29 @@ int sph_xyz_to_rangevoxel(const float *points, int m, int ndim, int v_res, int h
                           int use_log, int32_t *winner, float *feature, int32_t *depth, int32_t *thick,
                           int32_t *idx_out, void *stream);
 
+/* Replaces points_to_voxel_3d (include/point2voxel.h:412-512) together with the coordinate
+ * transforms of sphconv/utils/coord_transform.py:8-118: `points` [n,nfeat] float32 on the device
+ * (x, y, z, intensity first) are mapped to system coordinates (c0, c1, c2) --
+ *   system 0 spherical (r, phi, theta)   1 l-spherical (log r, phi, theta)
+ *          2 cylinder  (d, phi, z)       3 l-cylinder  (log d, phi, z)
+ *          4 hybrid    (d, phi, theta)   5 l-hybrid    (log d, phi, theta)
+ * -- and binned: bin_i = floor((c_i - lo_i) / vs_i), points with a bin outside [0, g_i) are skipped.
+ * Voxels are numbered in order of first appearance in the point list, keep their first max_points
+ * points, and every point from the one that would open voxel number max_voxels on is dropped, as
+ * in the reference's loop.  Outputs (all zero where unused): voxels [max_voxels, max_points, W]
+ * (append_mode 0: the point's nfeat values, W = nfeat; 1: those plus (c0, c1, c2), W = nfeat + 3;
+ * 2: (c0, c1, c2, intensity), W = nfeat), mask [max_voxels, max_points] (1.0 where a point sits),
+ * coors [max_voxels, 3] = (bin of c2, of c1, of c0), num_points [max_voxels], voxel_num [1] (device).
+ * cell_in (optional, [n] int64): take these cells ((bin2*g1 + bin1)*g0 + bin0, negative = skip)
+ * instead of computing them; cell_out (optional): receives the cells.  `workspace`: device memory
+ * of sph_points_to_voxel_workspace(n, g0, g1, g2) bytes, 256-byte aligned; nothing is allocated. */
+size_t sph_points_to_voxel_workspace(int n, int g0, int g1, int g2);
+int sph_points_to_voxel(const float *points, int n, int nfeat, int system, float lo0, float lo1, float lo2,
+                        float vs0, float vs1, float vs2, int g0, int g1, int g2, int max_points,
+                        int max_voxels, int append_mode, float *voxels, float *mask, int32_t *coors,
+                        int32_t *num_points, int32_t *voxel_num, const long long *cell_in,
+                        long long *cell_out, void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -281,3 +281,112 @@ def xyz2rangevoxel(points, v_res=64, h_res=512, d_res=512, v_range=(87.5, 103.4)
         thick[0, theta_idx[i], phi_idx[i]] = 1
     bins = np.stack([theta_idx, phi_idx, depth_idx], axis=1).astype(np.int32)
     return feature, depth, thick, bins, raw
+
+
+# ---- point cloud -> voxels (reference include/point2voxel.h, sphconv/utils/) ---------------
+
+_SYSTEMS = ("spherical", "l-spherical", "cylinder", "l-cylinder", "hybrid", "l-hybrid")
+
+
+def system_transform(points, coors_range, sphere_coors_range, coord_system):
+    """numpy restatement of sphconv/utils/coord_transform.py:8-118 for float32 points:
+    -> (system_points [N,4] float32 = (c0, c1, c2, intensity), system_range [6] float64)."""
+    pts = np.ascontiguousarray(points, dtype=np.float32)
+    x, y, z, intensity = pts[:, 0], pts[:, 1], pts[:, 2], pts[:, 3]
+    v, s = coors_range, sphere_coors_range
+    with np.errstate(all="ignore"):
+        x2y2 = x * x + y * y
+        r = np.sqrt(x2y2 + z * z)
+        d = np.sqrt(x2y2)
+        phi = np.arcsin(y / np.sqrt(x2y2))
+        theta = np.arccos(z / r)
+        rad = np.radians
+        if coord_system == "spherical":        # :8-24
+            c = (r, phi, theta); rng = [s[0], rad(s[1]), rad(s[2]), s[3], rad(s[4]), rad(s[5])]
+        elif coord_system == "l-spherical":    # :27-42
+            c = (np.log(r), phi, theta); rng = [np.log(s[0]), rad(s[1]), rad(s[2]), np.log(s[3]), rad(s[4]), rad(s[5])]
+        elif coord_system == "cylinder":       # :45-59
+            c = (d, phi, z); rng = [s[0], rad(s[1]), v[2], s[3], rad(s[4]), v[5]]
+        elif coord_system == "l-cylinder":     # :62-76
+            c = (np.log(d), phi, z); rng = [np.log(s[0]), rad(s[1]), v[2], np.log(s[3]), rad(s[4]), v[5]]
+        elif coord_system == "hybrid":         # :79-96
+            c = (d, phi, theta); rng = [s[0], rad(s[1]), rad(s[2]), s[3], rad(s[4]), rad(s[5])]
+        elif coord_system == "l-hybrid":       # :99-116
+            c = (np.log(d), phi, theta); rng = [np.log(s[0]), rad(s[1]), rad(s[2]), np.log(s[3]), rad(s[4]), rad(s[5])]
+        else:
+            raise ValueError("unknown coord_system %r" % (coord_system,))
+    return np.stack([c[0], c[1], c[2], intensity], 1).astype(np.float32), np.array(rng, dtype=np.float64)
+
+
+def voxel_cells(system_points, system_range, grid_size):
+    """Cell of every point as point2voxel.h:436-457 computes it (float32: the pybind11 template is
+    instantiated with the points' type, so range and voxel size are float32): (coor [N,3] int64 =
+    (idx of c2, idx of c1, idx of c0), valid [N] bool, float bins [N,3] in coordinate order)."""
+    f32 = np.float32
+    rng = np.asarray(system_range, dtype=np.float64).astype(np.float32)
+    g = [int(v) for v in grid_size]
+    vs = [f32((rng[3 + i] - rng[i]) / f32(g[i])) for i in range(3)]          # :436-439 (float32 / int -> float32)
+    sp = np.asarray(system_points, dtype=np.float32)
+    with np.errstate(all="ignore"):
+        fb = np.stack([(sp[:, i] - rng[i]) / vs[i] for i in range(3)], axis=1)  # float32
+    fl = np.floor(fb)
+    ok = np.isfinite(fb).all(1)
+    for i in range(3):
+        ok &= (fl[:, i] >= 0) & (fl[:, i] < g[i])
+    coor = np.where(ok[:, None], np.nan_to_num(fl, nan=0.0, posinf=0.0, neginf=0.0), 0).astype(np.int64)[:, ::-1]
+    return coor, ok, fb
+
+
+def voxelize_cells(points, system_points, coor, valid, max_points, max_voxels, append_mode=0):
+    """The sequential loop of points_to_voxel_3d (point2voxel.h:441-505) on given cells: voxels are
+    numbered in order of first appearance, keep their first ``max_points`` points, and the loop stops
+    at the point that would open voxel number ``max_voxels``.  Returns the reference's dict."""
+    pts = np.asarray(points, dtype=np.float32)
+    nfeat = pts.shape[1]
+    width = nfeat + 3 if append_mode == 1 else nfeat
+    voxels = np.zeros((max_voxels, max_points, width), np.float32)
+    mask = np.zeros((max_voxels, max_points), np.float32)
+    coors = np.zeros((max_voxels, 3), np.int32)
+    num = np.zeros((max_voxels,), np.int32)
+    table = {}
+    voxel_num = 0
+    for i in range(pts.shape[0]):
+        if not valid[i]:
+            continue
+        key = (int(coor[i, 0]), int(coor[i, 1]), int(coor[i, 2]))
+        vid = table.get(key, -1)
+        if vid == -1:
+            vid = voxel_num
+            if voxel_num >= max_voxels:
+                break
+            voxel_num += 1
+            table[key] = vid
+            coors[vid] = key
+        n = num[vid]
+        if n < max_points:
+            mask[vid, n] = 1
+            if append_mode == 0:
+                voxels[vid, n, :nfeat] = pts[i]
+            elif append_mode == 1:
+                voxels[vid, n, :nfeat] = pts[i]
+                voxels[vid, n, nfeat:nfeat + 3] = system_points[i, :3]
+            else:
+                voxels[vid, n, :3] = system_points[i, :3]
+                voxels[vid, n, 3] = pts[i, 3]
+            num[vid] += 1
+    return {"voxels": voxels, "coordinates": coors, "num_points_per_voxel": num,
+            "voxel_point_mask": mask.reshape(-1, max_points, 1), "voxel_num": voxel_num}
+
+
+def points_to_voxel_v2(points, coors_range, sphere_coors_range, max_points=1, max_voxels=30000,
+                       resolution_HWD=None, coord_system="spherical", append_mode=0):
+    """sphconv/utils/voxelize.py:126-214 with a resolution (the transform_funcs branch)."""
+    sp, rng = system_transform(points, coors_range, sphere_coors_range, coord_system)
+    coor, ok, _ = voxel_cells(sp, rng, resolution_HWD)
+    return voxelize_cells(points, sp, coor, ok, max_points, max_voxels, append_mode)
+
+
+def simple_voxel(voxels, num_points, num_input_features=4):
+    """SimpleVoxel.forward (sphconv/vfe.py:222-228): mean of a voxel's points."""
+    v = np.asarray(voxels, dtype=np.float32)
+    return (v[:, :, :num_input_features].sum(axis=1) / np.asarray(num_points, np.float32).reshape(-1, 1)).astype(np.float32)

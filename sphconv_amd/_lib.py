@@ -67,6 +67,9 @@ _SIGNATURES = {
     "sph_init_tensor_workspace": (_Z, [_I, _I, _I, _I, _I]),
     "sph_init_tensor": (_I, [_P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _Z, _P]),
     "sph_permute_rows": (_I, [_P, _P, _I, _I, _I, _P, _P]),
+    "sph_points_to_voxel_workspace": (_Z, [_I, _I, _I, _I]),
+    "sph_points_to_voxel": (_I, [_P, _I, _I, _I, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float, _I, _I,
+                                 _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "sph_xyz_to_rangevoxel": (_I, [_P, _I, _I, _I, _I, _I, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float,
                                    C.c_float, _I, _P, _P, _P, _P, _P, _P]),
     "sph_to_dense": (_I, [_P, _P, _P, _I, _I, _I, _I, _P, _P]),

@@ -1,0 +1,98 @@
+"""GPU parity of the point cloud -> voxel path (sph_points_to_voxel through sphconv_amd.voxelize /
+datagen) against the restatement of the reference (oracle.points_to_voxel_v2 ..., reference
+include/point2voxel.h:412-512, sphconv/utils/coord_transform.py, sphconv/vfe.py:210-228).
+
+The cells come out of float32 sqrt / acos / asin / log, whose device and numpy versions may differ
+in the last bit: cells must be equal except where the oracle's float bin is within 1e-3 of an
+integer (at most 0.1 % of the points may differ).  Given cells, everything else -- numbering in
+order of first appearance, the first max_points points, the stop at max_voxels -- is integer work
+and must be bit-exact, which is checked by feeding the oracle's cells to the device."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import sphconv_amd as sphconv
+from oracle import oracle as O
+from sphconv_amd.datagen import VoxelizationVFE, merge_batch_torch
+from sphconv_amd.voxelize import VoxelGeneratorV3, points_to_voxel_v2
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+KITTI = os.path.join(HERE, "golden", "kitti_000000_reduced.bin")   # reference test/000000.bin
+RANGE, SRANGE = [6, -40, -3, 70.4, 40, 1], [6, -45, 87.5, 70.4, 45, 100]
+
+
+def _compare(res, want):
+    m = want["voxel_num"]
+    assert res["voxel_num"] == m
+    for k in ("voxels", "coordinates", "num_points_per_voxel", "voxel_point_mask"):
+        assert np.array_equal(res[k].cpu().numpy(), want[k]), k
+
+
+@pytest.mark.parametrize("system", ["spherical", "l-spherical", "cylinder", "l-cylinder", "hybrid", "l-hybrid"])
+@pytest.mark.parametrize("grid,max_points,max_voxels,append_mode", [([512, 512, 64], 2, 24000, 0),
+                                                                    ([64, 96, 16], 3, 700, 1),
+                                                                    ([16, 16, 4], 5, 30000, 2)])
+def test_kitti_scan(system, grid, max_points, max_voxels, append_mode):
+    pts = np.fromfile(KITTI, dtype=np.float32).reshape(-1, 4)
+    sp, rng = O.system_transform(pts, RANGE, SRANGE, system)
+    coor, ok, fb = O.voxel_cells(sp, rng, grid)
+    cells = np.where(ok, (coor[:, 0] * grid[1] + coor[:, 1]) * grid[0] + coor[:, 2], -1)
+    # 1. cells computed on the device
+    res = points_to_voxel_v2(pts, None, RANGE, SRANGE, None, max_points, max_voxels, resolution_HWD=grid,
+                             coord_system=system, append_mode=append_mode, return_cells=True)
+    got = res["cells"].cpu().numpy()
+    with np.errstate(invalid="ignore"):
+        near = (np.abs(fb - np.rint(fb)) < 1e-3).any(1) | ~np.isfinite(fb).all(1)
+    differ = got != cells
+    assert (~differ | near).all() and differ.mean() <= 1e-3
+    # 2. integer part, bit-exact on the oracle's cells
+    want = O.voxelize_cells(pts, sp, coor, ok, max_points, max_voxels, append_mode)
+    res2 = points_to_voxel_v2(pts, None, RANGE, SRANGE, None, max_points, max_voxels, resolution_HWD=grid,
+                              coord_system=system, append_mode=append_mode, cells=torch.tensor(cells))
+    if append_mode == 0:
+        _compare(res2, want)
+    else:
+        # appended system coordinates are float32 transcendental results: compare those to 1e-6 relative
+        assert res2["voxel_num"] == want["voxel_num"]
+        for k in ("coordinates", "num_points_per_voxel", "voxel_point_mask"):
+            assert np.array_equal(res2[k].cpu().numpy(), want[k]), k
+        np.testing.assert_allclose(res2["voxels"].cpu().numpy(), want["voxels"], rtol=2e-6, atol=1e-6)
+    if not differ.any() and append_mode == 0:
+        _compare({k: v for k, v in res.items() if k != "cells"}, want)
+
+
+def test_small_and_degenerate_inputs():
+    pts = np.array([[20, 1, 0.2, 0.5], [20, 1, 0.2, 0.6], [0, 0, 3, 0.1], [0, 0, 0, 0.2], [1e3, 5, 1, 0.3],
+                    [30, -2, -1, 0.4], [20, 1, 0.2, 0.7]], np.float32)
+    for mv in (1, 2, 5):
+        res = points_to_voxel_v2(pts, None, RANGE, SRANGE, None, 2, mv, resolution_HWD=[8, 8, 4])
+        want = O.points_to_voxel_v2(pts, RANGE, SRANGE, 2, mv, [8, 8, 4], "spherical")
+        _compare(res, want)
+    res = points_to_voxel_v2(np.zeros((0, 4), np.float32), None, RANGE, SRANGE, None, 2, 10, resolution_HWD=[8, 8, 4])
+    assert res["voxel_num"] == 0 and float(res["voxels"].abs().sum()) == 0.0
+    with pytest.raises(ValueError):
+        points_to_voxel_v2(pts, None, RANGE, SRANGE, None, 2, 10, resolution_HWD=[8, 8, 4], coord_system="polar")
+
+
+def test_voxelization_vfe_feeds_the_convolution():
+    """datagen.VoxelizationVFE (reference test/common.py:30-59 builds its 'real' inputs with it):
+    file -> mean voxel features + coordinates -> SparseConvTensor -> convolution."""
+    shape_dwh = [16, 64, 64]
+    vvfe = VoxelizationVFE(resolution_HWD=shape_dwh[::-1])
+    voxels, coords = vvfe.generate(KITTI, torch.device("cuda:0"))
+    pts = np.fromfile(KITTI, dtype=np.float32).reshape(-1, 4)
+    want = O.points_to_voxel_v2(pts, RANGE, SRANGE, 2, 24000, shape_dwh[::-1], "spherical")
+    m = want["voxel_num"]
+    if voxels.shape[0] == m and np.array_equal(coords.cpu().numpy(), want["coordinates"][:m]):
+        mean = O.simple_voxel(want["voxels"][:m], want["num_points_per_voxel"][:m])
+        np.testing.assert_allclose(voxels.cpu().numpy(), mean, rtol=1e-6, atol=1e-7)
+    assert abs(voxels.shape[0] - m) <= max(2, m // 500)
+    assert (coords.cpu().numpy().max(0) < shape_dwh).all()
+    batch = merge_batch_torch([{"voxels": voxels, "coordinates": coords}] * 2)
+    assert batch["coordinates"].shape == (2 * voxels.shape[0], 4) and batch["coordinates"][:, 0].max() == 1
+    x = sphconv.SparseConvTensor(batch["voxels"], shape_dwh, 2, indices=batch["coordinates"])
+    y = sphconv.SubMConv3d(4, 8, 3).cuda()(x)
+    assert y.feature.shape == (2 * voxels.shape[0], 8) and torch.isfinite(y.feature).all()
