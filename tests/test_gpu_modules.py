@@ -116,3 +116,43 @@ def test_rangevoxel_bridge():
     assert torch.equal(rv.dense(), x.dense().permute(0, 1, 4, 2, 3))
     with pytest.raises(AssertionError):
         sphconv.RangeVoxel(rv.feature, rv.depth, rv.thick, (B, C + 1, D_, H_, W_))
+
+
+@pytest.mark.parametrize("subm,stride,padding", [(True, 1, 1), (False, 2, 1)])
+def test_real_scan_through_the_whole_path(subm, stride, padding):
+    """The reference's 'real' inputs (test/common.py:30-59: scan file -> voxels -> mean VFE, batch of
+    two, channels repeated to 8; used at test_grad.py:192-299, 428-563): forward, dgrad and wgrad of one
+    layer against torch's dense conv3d autograd in float64."""
+    import os
+    from sphconv_amd.datagen import VoxelizationVFE, merge_batch_torch
+    kitti = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "kitti_000000_reduced.bin")
+    shape, B, ic, oc = [8, 32, 32], 2, 8, 16                       # spatial_shape_DWH
+    vvfe = VoxelizationVFE(resolution_HWD=shape[::-1])
+    voxels, coords = vvfe.generate(kitti, torch.device(G.DEV))
+    ex = merge_batch_torch([{"voxels": voxels, "coordinates": coords}] * B)
+    feat = ex["voxels"].repeat((1, 2))[:, :ic].contiguous()
+    idx = ex["coordinates"].contiguous()
+    assert idx.shape[0] > 1000
+    cls = sphconv.SubMConv3d if subm else sphconv.SparseConv3d
+    conv = cls(ic, oc, 3, stride=stride, padding=padding, bias=False).to(G.DEV)
+    f = feat.clone().requires_grad_(True)
+    x = sphconv.SparseConvTensor(f, shape, B, indices=idx)
+    dense_y = conv(x).dense()
+    w64 = conv.weight.detach().double().cpu().requires_grad_(True)
+    f64 = feat.detach().double().cpu().requires_grad_(True)
+    c = idx.long().cpu()
+    d_in = torch.zeros((B, *shape, ic), dtype=torch.float64).index_put((c[:, 0], c[:, 1], c[:, 2], c[:, 3]), f64)
+    ref = torch.nn.functional.conv3d(d_in.permute(0, 4, 1, 2, 3), w64.permute(4, 3, 0, 1, 2), None, stride, padding)
+    if subm:
+        mask = torch.zeros((B, 1, *shape), dtype=torch.float64)
+        mask[c[:, 0], 0, c[:, 1], c[:, 2], c[:, 3]] = 1
+        ref = ref * mask
+    scale = float(ref.detach().abs().max())
+    torch.testing.assert_close(dense_y.detach().double().cpu(), ref.detach(), rtol=1e-4, atol=1e-5 * scale)
+    up = torch.randn(ref.shape, dtype=torch.float64, generator=torch.Generator().manual_seed(0))
+    up = up * (mask if subm else (ref.detach().abs().sum(1, keepdim=True) != 0))
+    (ref * up).sum().backward()
+    (dense_y * up.to(G.DEV).float()).sum().backward()
+    torch.testing.assert_close(f.grad.double().cpu(), f64.grad, rtol=1e-4, atol=1e-5 * float(f64.grad.abs().max()))
+    torch.testing.assert_close(conv.weight.grad.double().cpu(), w64.grad, rtol=1e-4,
+                               atol=1e-5 * float(w64.grad.abs().max()))
