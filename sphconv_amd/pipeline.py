@@ -1,0 +1,105 @@
+"""Several scans in flight: rule generation + forward of one submanifold layer for a
+stream of independent LiDAR scans, each scan on one of a few HIP streams.
+
+No reference counterpart (the reference launches everything on the legacy default
+stream, rule_conv.cu:139,333).  One 100k-voxel scan fills neither kernel's grid (a few
+hundred workgroups, one wave per SIMD), so the rule kernel of the next scan can run
+beside the convolution of the current one; the work per scan is unchanged.  All device
+memory (rule books, packed weights, outputs) is allocated once, per stream slot.
+"""
+import ctypes as C
+from typing import List, Sequence, Tuple
+
+import torch
+
+from . import _lib as L
+from .rulebook import _Buffers, _check_index_tensors
+
+
+class ScanPipeline:
+    """``submit(feature, z_idx, z_ptr)`` enqueues rules + forward of one scan on the next
+    stream slot and returns ``(out, slot)``; ``out`` [n, oC] is a view of that slot's output
+    buffer and is overwritten when the slot comes round again (after ``streams`` submits).
+    Call ``wait(slot)`` (or ``synchronize()``) before reading it on another stream."""
+
+    def __init__(self, weight: torch.Tensor, batch: int, shape: Sequence[int], kernel: Sequence[int] = (3, 3, 3),
+                 max_voxels: int = 1 << 18, streams: int = 3):
+        if weight.dim() == 5:
+            weight = weight.reshape(-1, weight.shape[3], weight.shape[4])
+        if weight.dim() != 3 or not weight.is_cuda:
+            raise L.SphconvError("weight must be a GPU tensor [KV,iC,oC] or [K0,K1,K2,iC,oC]")
+        self.weight = weight.detach().contiguous()
+        self.kv, self.ic, self.oc = (int(v) for v in self.weight.shape)
+        self.kernel = [int(k) for k in kernel]
+        if self.kernel[0] * self.kernel[1] * self.kernel[2] != self.kv:
+            raise L.SphconvError("weight holds %d offsets, kernel %s has %d" % (self.kv, self.kernel,
+                                 self.kernel[0] * self.kernel[1] * self.kernel[2]))
+        self.batch, self.shape = int(batch), [int(v) for v in shape]
+        self.max_voxels = int(max_voxels)
+        self.dt = L.dtype_code(self.weight.dtype)
+        dev = self.weight.device
+        lib = L.lib()
+        pad = [k // 2 for k in self.kernel]
+        self._geom = L.make_geom(self.batch, self.shape, self.shape, self.kernel, (1, 1, 1), pad)
+        nbytes = lib.sph_weight_packed_bytes(self.dt, self.kv, self.ic, self.oc)
+        if nbytes == 0:
+            raise L.SphconvError("cannot pack weight of shape %s" % (tuple(self.weight.shape),))
+        self._epi = L.Epilogue(None, None, 0)
+        self._streams = [torch.cuda.Stream(device=dev) for _ in range(int(streams))]
+        self._books = [_Buffers(self.max_voxels, self.kv, dev) for _ in self._streams]
+        self._packed = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in self._streams]
+        self._out = [torch.empty((self.max_voxels, self.oc), dtype=self.weight.dtype, device=dev) for _ in self._streams]
+        self._done = [torch.cuda.Event() for _ in self._streams]
+        self._next = 0
+        self._lib = lib
+
+    @property
+    def streams(self) -> int:
+        return len(self._streams)
+
+    def submit(self, feature: torch.Tensor, z_idx: torch.Tensor, z_ptr: torch.Tensor,
+               wait_inputs: bool = True) -> Tuple[torch.Tensor, int]:
+        """``wait_inputs=False`` skips making the slot's stream wait for the caller's current stream:
+        only for inputs that are already complete (e.g. produced before a synchronisation, or on
+        ``stream_of(slot)`` itself)."""
+        n = int(z_idx.shape[0])
+        if n > self.max_voxels:
+            raise L.SphconvError("scan of %d voxels, pipeline sized for %d" % (n, self.max_voxels))
+        if feature.shape != (n, self.ic) or feature.dtype != self.weight.dtype or not feature.is_contiguous():
+            raise L.SphconvError("feature must be contiguous [%d,%d] %s" % (n, self.ic, self.weight.dtype))
+        _check_index_tensors(z_idx, z_ptr, self.batch, self.shape)
+        slot = self._next
+        self._next = (slot + 1) % len(self._streams)
+        side = self._streams[slot]
+        if wait_inputs:
+            side.wait_stream(torch.cuda.current_stream())   # the inputs were produced on the caller's stream
+        st = side.cuda_stream
+        book = self._books[slot]
+        book._struct.rows = n                                 # the slot's buffers hold up to max_voxels rows
+        lib, w = self._lib, self.weight
+        rc = lib.sph_rules_build_pack(z_idx.data_ptr(), z_ptr.data_ptr(), n, z_idx.data_ptr(), z_ptr.data_ptr(), n,
+                                      C.byref(self._geom), 0, C.byref(book._struct), self.dt, w.data_ptr(), self.kv,
+                                      self.ic, self.oc, self.ic * self.oc, self.oc, 1,
+                                      self._packed[slot].data_ptr(), st)
+        if rc == 0:
+            rc = lib.sph_conv_apply(self.dt, feature.data_ptr(), n, self.ic, self._packed[slot].data_ptr(), self.oc,
+                                    C.byref(book._struct), C.byref(self._epi), self._out[slot].data_ptr(), st)
+        if rc:
+            L.check(rc)
+        self._done[slot].record(side)
+        return self._out[slot][:n], slot
+
+    def next_slot(self) -> int:
+        return self._next
+
+    def stream_of(self, slot: int) -> torch.cuda.Stream:
+        """The slot's stream, for producers that want to enqueue a scan's inputs where it will be used."""
+        return self._streams[slot]
+
+    def wait(self, slot: int):
+        """Makes the caller's current stream wait for the scan last submitted to ``slot``."""
+        torch.cuda.current_stream().wait_event(self._done[slot])
+
+    def synchronize(self):
+        for s in self._streams:
+            s.synchronize()

@@ -156,3 +156,38 @@ def test_real_scan_through_the_whole_path(subm, stride, padding):
     torch.testing.assert_close(f.grad.double().cpu(), f64.grad, rtol=1e-4, atol=1e-5 * float(f64.grad.abs().max()))
     torch.testing.assert_close(conv.weight.grad.double().cpu(), w64.grad, rtol=1e-4,
                                atol=1e-5 * float(w64.grad.abs().max()))
+
+
+def test_scan_pipeline_matches_the_plain_path():
+    """ScanPipeline (scans in flight on several HIP streams) returns the bits of
+    get_rulebook_subm + rule_conv for every scan, whatever slot it lands in."""
+    from sphconv_amd import sphconv_cuda as ext
+    from sphconv_amd.pipeline import ScanPipeline
+    from sphconv_amd.rulebook import RuleBook
+    B, shape, ic, oc = 2, [10, 24, 16], 16, 32
+    rng = np.random.default_rng(3)
+    w = G.t((rng.standard_normal((3, 3, 3, ic, oc)) * 0.1).astype(np.float32)).half()
+    pipe = ScanPipeline(w, B, shape, max_voxels=4096, streams=3)
+    assert pipe.streams == 3
+    scans = []
+    for s in range(7):                                     # more scans than slots, different sizes
+        idx, feat = _inputs(10 + s, B, shape, ic, p=0.1 + 0.05 * s)
+        x = sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx))
+        book = RuleBook.build_subm(x.z_idx, x.z_ptr, B, shape, [3, 3, 3])
+        want = ext.rule_conv(x.feature, w.view(27, ic, oc), book, None, x.feature.shape[0])
+        scans.append((x, want))
+    torch.cuda.synchronize()
+    pending = []
+    for i, (x, want) in enumerate(scans):
+        out, slot = pipe.submit(x.feature, x.z_idx, x.z_ptr)
+        pending.append((out, slot, want))
+        if len(pending) == pipe.streams:                   # read a slot before it is used again
+            o, sl, wnt = pending.pop(0)
+            pipe.wait(sl)
+            assert torch.equal(o, wnt)
+    pipe.synchronize()
+    for o, sl, wnt in pending:
+        assert torch.equal(o, wnt)
+    with pytest.raises(sphconv.SphconvError):
+        big = torch.zeros((5000, ic), dtype=torch.float16, device=G.DEV)
+        pipe.submit(big, torch.zeros(5000, dtype=torch.int32, device=G.DEV), scans[0][0].z_ptr)
