@@ -45,6 +45,9 @@ def parse():
     ap.add_argument("--backward", action="store_true",
                     help="also time dgrad (transposed rule book + kernel) and wgrad of the same layer; "
                          "reported under 'kernels', not part of 'value'")
+    ap.add_argument("--encoder", action="store_true",
+                    help="also time configuration 4 (four-stage encoder, batch 4, fp16, rules regenerated every "
+                         "pass) end to end; reported under 'encoder_stack', not part of 'value'")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 256 MiB device-to-device copies (a kernel of known HBM traffic, "
@@ -103,6 +106,43 @@ def cpu_baseline(d, ic, oc, budget_s, seed):
                       "fp32, tile 2x2, tile_n_max %d, dropped pairs %d"
                       % (len(times), n, rg * 1e3, fw * 1e3, n_max, times[0][2]),
             "rulegen_ms": rg * 1e3, "forward_ms": fw * 1e3}
+
+
+def encoder_stack_ms(torch, seed, iters):
+    """Configuration 4: batch of four scans through the four-stage encoder (12 convolutions, each with
+    BatchNorm(eval) + ReLU), every pass regenerates all rule books; fused tails and separate modules."""
+    import numpy as np
+    import sphconv_amd as sphconv
+    from sphconv_amd.synth import encoder_stack, make_config
+    d = make_config(4, seed=seed)
+    shape, B = d["spatial_shape"], d["batch"]
+    n = int(d["z_idx"].shape[0])
+    dev = "cuda:0"
+    rng = np.random.default_rng(seed)
+    feat = torch.tensor(rng.standard_normal((n, 16)), dtype=torch.float32, device=dev).half()
+    z_idx, z_ptr = torch.tensor(d["z_idx"], device=dev), torch.tensor(d["z_ptr"], device=dev)
+    net = encoder_stack(16, (16, 32, 64, 64), seed=seed).to(dev).half()
+    res = {"batch": B, "voxels_in": n}
+
+    def one():
+        with torch.no_grad():
+            return net(sphconv.SparseConvTensor(feat, shape, B, z_idx=z_idx, z_ptr=z_ptr))
+
+    for fused in (True, False):
+        net.fuse_eval = fused
+        for _ in range(3):
+            y = one()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            y = one()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / iters * 1e3
+        res["fused_ms_per_batch" if fused else "separate_modules_ms_per_batch"] = ms
+        if fused:
+            res["ms_per_scan"] = ms / B
+            res["voxels_out"] = int(y.feature.shape[0])
+    return res
 
 
 def main():
@@ -235,6 +275,8 @@ def main():
                     "conv_TFLOPs": conv_flops / (conv_ms * 1e-3) / 1e12, **extra},
         "roofline": roofline,
     }
+    if args.encoder:
+        result["encoder_stack"] = encoder_stack_ms(torch, args.seed, 20)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(d, ic, oc, args.cpu_seconds, args.seed)
     print(json.dumps(result))

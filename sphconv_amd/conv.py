@@ -6,6 +6,7 @@ from typing import List, Optional
 import torch
 import torch.nn as nn
 
+from . import sphconv_cuda as ext
 from .functional import ConvFunction
 from .modules import SphModule
 from .rulebook import RuleBook
@@ -111,7 +112,10 @@ class Conv3d(Convolution):
             input.rule_cache[self.indice_key] = entry
         return entry, packed
 
-    def forward(self, input: SparseConvTensor) -> SparseConvTensor:
+    def forward(self, input: SparseConvTensor, epilogue=None) -> SparseConvTensor:
+        """``epilogue`` = (scale [oC] fp32 or None, shift [oC] fp32 or None, relu): applied to the
+        accumulators before the store, inference only (no autograd through it; no reference
+        counterpart)."""
         assert self.in_channels == input.C, \
             "input channel does not match Expect: {}, got {}".format(self.in_channels, input.C)
         in_shape = [input.D, input.W, input.H]
@@ -120,8 +124,16 @@ class Conv3d(Convolution):
         weight = self.weight.view(-1, self.in_channels, self.out_channels)
         (oz_idx, oz_ptr, book, rule_size, tile_grid_shape), packed = self._rules(input, out_shape, weight)
         self.rule_book = book if isinstance(book, RuleBook) else None
-        out_feature = ConvFunction.apply(input.feature, weight, book, rule_size, tile_grid_shape,
-                                         oz_idx.shape[0], packed)
+        if epilogue is not None:
+            if torch.is_grad_enabled() and (weight.requires_grad or input.feature.requires_grad):
+                raise RuntimeError("a fused epilogue has no backward: call under torch.no_grad()")
+            scale, shift, relu = epilogue
+            w = weight if weight.dtype == input.feature.dtype else weight.to(input.feature.dtype)
+            out_feature = ext.rule_conv(input.feature, w, book, rule_size, oz_idx.shape[0], scale, shift,
+                                        bool(relu), packed if w is weight else None)
+        else:
+            out_feature = ConvFunction.apply(input.feature, weight, book, rule_size, tile_grid_shape,
+                                             oz_idx.shape[0], packed)
         out = SparseConvTensor(out_feature, out_shape, input.B, z_ptr=oz_ptr, z_idx=oz_idx)
         out.rule_cache = input.rule_cache
         return out

@@ -20,10 +20,42 @@ def is_sparse_conv(module) -> bool:
     return isinstance(module, Convolution)
 
 
+def _bn_affine(bn: nn.BatchNorm1d):
+    """Evaluation-mode BatchNorm1d as y = x*scale + shift (fp32 [C]); computed once per state of
+    the module's tensors (their version counters) and kept on the module."""
+    tensors = (bn.running_mean, bn.running_var, bn.weight, bn.bias)
+    key = tuple((t.data_ptr(), t._version, t.dtype) if t is not None else None for t in tensors) + (bn.eps,)
+    cached = getattr(bn, "_sph_affine", None)
+    if cached is not None and cached[0] == key:
+        return cached[1], cached[2]
+    scale, shift = _bn_affine_now(bn)
+    bn._sph_affine = (key, scale, shift)
+    return scale, shift
+
+
+def _bn_affine_now(bn: nn.BatchNorm1d):
+    var = bn.running_var.float()
+    scale = torch.rsqrt(var + bn.eps)
+    if bn.weight is not None:
+        scale = scale * bn.weight.float()
+    shift = -bn.running_mean.float() * scale
+    if bn.bias is not None:
+        shift = shift + bn.bias.float()
+    return scale.contiguous(), shift.contiguous()
+
+
 class Sequential(SphModule):
     """Sequential container over sparse-conv and ordinary modules
     (modules.py:43-128).  Accepts positional modules, one OrderedDict, or keyword
-    modules."""
+    modules.
+
+    With gradients disabled, a convolution followed by an evaluation-mode
+    ``BatchNorm1d`` and/or a ``ReLU`` runs as one kernel: the affine map and the
+    clamp are applied to the fp32 accumulators before the store (no reference
+    counterpart: modules.py:124-125 runs them as separate passes over ``.feature``).
+    ``fuse_eval = False`` switches this off."""
+
+    fuse_eval = True
 
     def __init__(self, *args, **kwargs):
         super().__init__()
@@ -55,13 +87,41 @@ class Sequential(SphModule):
                 raise KeyError("name exists")
         self.add_module(name, module)
 
+    def _fusable_tail(self, mods, i):
+        """(number of modules after mods[i] that fold into its store, BatchNorm1d or None, relu)."""
+        conv = mods[i]
+        if not (self.fuse_eval and is_sparse_conv(conv)) or torch.is_grad_enabled():
+            return 0, None, False
+        if conv.weight.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+            return 0, None, False
+        n, bn, relu = 0, None, False
+        nxt = mods[i + 1] if i + 1 < len(mods) else None
+        if (type(nxt) is nn.BatchNorm1d and not nxt.training and nxt.running_mean is not None
+                and nxt.num_features == conv.out_channels):
+            bn, n = nxt, 1
+            nxt = mods[i + 2] if i + 2 < len(mods) else None
+        if type(nxt) is nn.ReLU:
+            relu, n = True, n + 1
+        return n, bn, relu
+
     def forward(self, input):
         from .tensor import SparseConvTensor
-        for name, module in self._modules.items():
+        mods = list(self._modules.items())
+        only = [m for _, m in mods]
+        skip = 0
+        for i, (name, module) in enumerate(mods):
+            if skip:
+                skip -= 1
+                continue
             if is_sph_module(module):
                 assert isinstance(input, SparseConvTensor)
                 with torch.autograd.profiler.record_function("sphconv:{}:{}".format(type(module).__name__, name)):
-                    input = module(input)
+                    skip, bn, relu = self._fusable_tail(only, i)
+                    if skip:
+                        scale, shift = _bn_affine(bn) if bn is not None else (None, None)
+                        input = module(input, epilogue=(scale, shift, relu))
+                    else:
+                        input = module(input)
             elif isinstance(input, SparseConvTensor):
                 input.feature = module(input.feature)
             else:

@@ -91,3 +91,35 @@ def make_config(cfg: int, seed: int = 0, batch: int = None):
     idx, z_idx, z_ptr = _csr_from_occupancy(occ)
     return {"indices": idx, "z_idx": z_idx, "z_ptr": z_ptr,
             "spatial_shape": list(shape), "batch": B}
+
+
+def encoder_stack(in_channels: int = 16, widths=(16, 32, 64, 64), seed: int = 0, neighbours: float = 8.0):
+    """The four-stage middle encoder of benchmark configuration 4 as a ``Sequential``:
+    per stage two submanifold 3x3x3 convolutions sharing one rule book, then a 3x3x3
+    convolution of stride 2 / padding 1, each followed by BatchNorm1d (evaluation mode,
+    random affine and statistics) and ReLU.  Weights are normal with the variance that keeps
+    activations of a voxel with ``neighbours`` active neighbours at unit scale."""
+    import torch
+    from torch import nn
+
+    from .conv import SparseConv3d, SubMConv3d
+    from .modules import Sequential
+
+    gen = torch.Generator().manual_seed(seed)
+    layers = []
+    c_in = in_channels
+    for s, c in enumerate(widths):
+        for conv in (SubMConv3d(c_in, c, 3, indice_key="subm%d" % s), SubMConv3d(c, c, 3, indice_key="subm%d" % s),
+                     SparseConv3d(c, c, 3, stride=2, padding=1)):
+            with torch.no_grad():
+                std = (2.0 / (neighbours * conv.in_channels)) ** 0.5
+                conv.weight.copy_(torch.randn(conv.weight.shape, generator=gen) * std)
+            bn = nn.BatchNorm1d(c)
+            with torch.no_grad():
+                bn.weight.copy_(0.75 + 0.5 * torch.rand(c, generator=gen))
+                bn.bias.copy_(0.1 * torch.randn(c, generator=gen))
+                bn.running_mean.copy_(0.1 * torch.randn(c, generator=gen))
+                bn.running_var.copy_(0.75 + 0.5 * torch.rand(c, generator=gen))
+            layers += [conv, bn, nn.ReLU()]
+        c_in = c
+    return Sequential(*layers).eval()

@@ -7,6 +7,8 @@ import torch
 import helpers as H
 import gpu_helpers as G
 import sphconv_amd as sphconv
+from oracle import oracle as O
+from sphconv_amd.synth import make_config
 
 pytestmark = pytest.mark.gpu
 
@@ -191,3 +193,84 @@ def test_scan_pipeline_matches_the_plain_path():
     with pytest.raises(sphconv.SphconvError):
         big = torch.zeros((5000, ic), dtype=torch.float16, device=G.DEV)
         pipe.submit(big, torch.zeros(5000, dtype=torch.int32, device=G.DEV), scans[0][0].z_ptr)
+
+
+def test_fused_eval_tail_equals_separate_modules():
+    """conv + BatchNorm1d(eval) + ReLU as one kernel against the same modules run one by one."""
+    from sphconv_amd.synth import encoder_stack
+    B, shape = 2, [16, 32, 16]
+    idx, feat = _inputs(5, B, shape, 16)
+    net = encoder_stack(16, (16, 32), seed=1).to(G.DEV).half()
+    x = sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx))
+    with torch.no_grad():
+        fused = net(x)
+        net.fuse_eval = False
+        x2 = sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx))
+        plain = net(x2)
+    assert torch.equal(fused.z_idx, plain.z_idx) and torch.equal(fused.z_ptr, plain.z_ptr)
+    assert float(plain.feature.float().abs().mean()) > 1e-2
+    # the separate modules round to fp16 after the convolution and again after the batch norm
+    torch.testing.assert_close(fused.feature.float(), plain.feature.float(), rtol=2e-2, atol=2e-2)
+    # the affine map kept on a BatchNorm module follows in-place changes of its tensors
+    net.fuse_eval = True
+    with torch.no_grad():
+        net[1].weight.mul_(-1.5)
+        net[1].running_mean.add_(0.25)
+        fused2 = net(sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx)))
+        net.fuse_eval = False
+        plain2 = net(sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx)))
+        net[1].weight.div_(-1.5)
+        net[1].running_mean.sub_(0.25)
+    assert not torch.allclose(plain2.feature.float(), plain.feature.float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(fused2.feature.float(), plain2.feature.float(), rtol=2e-2, atol=2e-2)
+    # with gradients enabled nothing is fused (autograd needs the separate modules)
+    net.fuse_eval = True
+    x3 = sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx))
+    y3 = net(x3)
+    assert y3.feature.requires_grad
+    torch.testing.assert_close(y3.feature.detach().float(), plain.feature.float(), rtol=2e-3, atol=2e-3)
+
+
+def test_config4_encoder_full_size_layer_by_layer():
+    """BASELINE configuration 4 (batch 4, grid 64x2048x64, four stages of two submanifold and one
+    strided convolution, BatchNorm + ReLU fused, fp16): every layer's output against the C oracle
+    applied to that layer's own input, rules included."""
+    from sphconv_amd.synth import encoder_stack
+    d = make_config(4, seed=0)
+    shape, B = d["spatial_shape"], d["batch"]
+    n = d["z_idx"].shape[0]
+    rng = np.random.default_rng(4)
+    feat = torch.tensor(rng.standard_normal((n, 16)), dtype=torch.float32).half()
+    net = encoder_stack(16, (16, 32, 64, 64), seed=4).to(G.DEV).half()
+    x = sphconv.SparseConvTensor(feat.to(G.DEV), shape, B, z_idx=G.t(d["z_idx"]), z_ptr=G.t(d["z_ptr"]))
+    mods = list(net)
+    with torch.no_grad():
+        for i in range(0, len(mods), 3):
+            conv, bn = mods[i], mods[i + 1]
+            z_idx, z_ptr = x.z_idx.cpu().numpy(), x.z_ptr.cpu().numpy()
+            f_in = x.feature.float().cpu().numpy()
+            in_shape = [x.D, x.W, x.H]
+            y = sphconv.Sequential(*mods[i:i + 3])(x)
+            if conv.subm:
+                oshape = in_shape
+                ora = O.get_rules_subm(z_idx, z_ptr, B, in_shape, oshape, [3, 3, 3], [1, 1, 1], [1, 1, 1], n_max=512)
+            else:
+                oshape = H.out_shape_of(in_shape, [3, 3, 3], [2, 2, 2], [1, 1, 1])
+                ora = O.get_rules(z_idx, z_ptr, B, in_shape, oshape, [3, 3, 3], [2, 2, 2], [1, 1, 1], n_max=512)
+            oz_idx, oz_ptr, rules, rule_size, dropped = ora
+            assert dropped == 0
+            assert [y.D, y.W, y.H] == list(oshape)
+            assert np.array_equal(y.z_idx.cpu().numpy(), oz_idx) and np.array_equal(y.z_ptr.cpu().numpy(), oz_ptr)
+            w = conv.weight.detach().float().cpu().numpy().reshape(27, conv.in_channels, conv.out_channels)
+            acc = O.rule_conv(f_in, w, rules, rule_size, oz_idx.shape[0])
+            scale = (bn.weight.float() / torch.sqrt(bn.running_var.float() + bn.eps)).cpu().numpy()
+            shift = (bn.bias.float() - bn.running_mean.float() * bn.weight.float()
+                     / torch.sqrt(bn.running_var.float() + bn.eps)).cpu().numpy()
+            want = np.maximum(acc * scale[None, :] + shift[None, :], 0.0)
+            got = y.feature.float().cpu().numpy()
+            assert got.shape == want.shape
+            # fp32 accumulate, one rounding to fp16 (tolerance of the task: rtol 1e-2, atol 1e-3)
+            assert (np.abs(got - want) <= 2.0 ** -9 * np.abs(want) + 1e-3).all(), i
+            assert 0.2 < (want > 0).mean() < 0.9 and 1e-2 < np.abs(want).mean() < 1e2, (i, np.abs(want).mean())
+            x = y
+    assert [x.D, x.W, x.H] == [4, 128, 4] and x.feature.shape[1] == 64
