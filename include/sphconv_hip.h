@@ -121,17 +121,20 @@ int sph_rules_build_pack(const int32_t *z_idx, const int32_t *z_ptr, int in_rows
 
 /* Replaces the output-coordinate half of get_rules (rules.cu:417-443, 461-462),
  * in two steps because the caller must size oz_idx:
- *  1. sph_outcoords_count: per-column output counts into oz_ptr (used as
- *     scratch), block partial sums into block_sums [sph_outcoords_blocks(g)],
- *     their exclusive scan in place, and the total in *total_dev (device int).
- *  2. after reading *total_dev: sph_outcoords_fill writes the final oz_ptr
- *     (inclusive scan) and oz_idx (ascending within a column). */
+ *  1. sph_outcoords_count: per-column output counts into oz_ptr, their inclusive scan in
+ *     place (`scratch`: 8-byte aligned device memory of sph_outcoords_scratch_ints(g) int32,
+ *     holding the scan's temporary storage and, when O[2] <= 64, each column's 64-bit mask
+ *     of active bins), and the total in *total_dev (device int).
+ *  2. after reading *total_dev: sph_outcoords_fill, given the same scratch and oz_ptr, writes
+ *     oz_idx (ascending within a column).
+ * sph_outcoords_blocks(g) = ceil(columns / 256), the grid of the fill kernel. */
 int sph_outcoords_blocks(const sph_geom *g);
+int sph_outcoords_scratch_ints(const sph_geom *g);
 int sph_outcoords_count(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
-                        const sph_geom *g, int32_t *oz_ptr, int32_t *block_sums,
+                        const sph_geom *g, int32_t *oz_ptr, int32_t *scratch,
                         int32_t *total_dev, void *stream);
 int sph_outcoords_fill(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
-                       const sph_geom *g, const int32_t *block_sums, int32_t *oz_ptr,
+                       const sph_geom *g, const int32_t *scratch, int32_t *oz_ptr,
                        int32_t *oz_idx, int out_rows, void *stream);
 
 /* Conversions between the rule book and the reference's padded tensors

@@ -54,6 +54,7 @@ _SIGNATURES = {
     "sph_rules_build_pack": (_I, [_P, _P, _I, _P, _P, _I, C.POINTER(Geom), _I, C.POINTER(Book), _I, _P, _I, _I, _I, _L, _L,
                                   _L, _P, _P]),
     "sph_outcoords_blocks": (_I, [C.POINTER(Geom)]),
+    "sph_outcoords_scratch_ints": (_I, [C.POINTER(Geom)]),
     "sph_outcoords_count": (_I, [_P, _P, _I, C.POINTER(Geom), _P, _P, _P, _P]),
     "sph_outcoords_fill": (_I, [_P, _P, _I, C.POINTER(Geom), _P, _P, _P, _I, _P]),
     "sph_rules_to_padded_count": (_I, [C.POINTER(Book), _P, C.POINTER(Geom), _I, _I, _P, _P, _P]),

@@ -6,6 +6,11 @@
 #include "common.h"
 #include "pack.h"
 
+#include <cstring>
+
+#include <rocprim/device/device_scan.hpp>
+#include <rocprim/functional.hpp>
+
 namespace {
 
 constexpr int kThreads = 256;
@@ -198,8 +203,13 @@ struct BuildArgs {
     // optional passenger: workgroups behind the tile workgroups pack a weight (total == 0: none)
     SphPackJob pack;
     int tile_blocks;
+    // gathered-side fibers are long (several entries on average) and their bins fit a 64-bit mask:
+    // join through per-column occupancy masks instead of walking a fiber once per row
+    int long_fibers;
 };
 
+constexpr int kMaskCols = 32;  // distinct columns of a tile the mask join provides for
+constexpr int kMaskWalk = 16;  // fiber entries fetched together when a mask is built
 constexpr int kJoinItems = 5; // (row, k0, k1) items a thread joins per pass, all loads of a pass in flight together
 
 template <bool TRANSPOSED>
@@ -271,11 +281,108 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     }
     __syncthreads();
 
+    // 2a. join through masks (long fibers).  The tile's rows share few columns, and every row of
+    // a column would walk the same K0*K1 fibers of the other grid: walk each (column, k0, k1)
+    // fiber once into a 64-bit occupancy mask, then every (row, k0, k1, k2) is a bit test and a
+    // popcount (position inside the sorted fiber).  A fiber that is not strictly ascending or
+    // leaves the 64 bins sends the whole tile to the general join below.
+    bool by_masks = false;
+    if (a.long_fibers) {
+        unsigned long long *s_cmask = (unsigned long long *)(s_nbr + R * KV); // [K01][ncols], ncols <= kMaskCols
+        int *s_cstart = (int *)(s_cmask + kMaskCols * K01);
+        __shared__ int s_cj[R], s_rep[R], s_bad;
+        __shared__ unsigned long long s_bal[R / kWave];
+        const int lane = tid & (kWave - 1), wave = tid / kWave;
+        if (tid == 0) s_bad = 0;
+        bool head = false;
+        if (tid < R) {
+            head = tid < nrows && s_col[tid] >= 0 && (tid == 0 || s_col[tid] != s_col[tid - 1]);
+            const unsigned long long bal = __ballot(head);
+            if (lane == 0) s_bal[wave] = bal;
+        }
+        __syncthreads();
+        int ncols = 0;
+        for (int w = 0; w < R / kWave; w++) ncols += __popcll(s_bal[w]);
+        if (tid < R) {
+            int incl = __popcll(s_bal[wave] & ((2ull << lane) - 1ull)); // heads at or before this row
+            for (int w = 0; w < wave; w++) incl += __popcll(s_bal[w]);
+            const int cj = (tid < nrows && s_col[tid] >= 0) ? incl - 1 : -1;
+            s_cj[tid] = cj;
+            if (head) s_rep[cj] = tid;
+        }
+        __syncthreads();
+        if (ncols > kMaskCols) ncols = 0; // short fibers after all: general join
+        for (int it = tid; it < ncols * K01; it += kThreads) {
+            const int k01 = it / ncols, cj = it - k01 * ncols;
+            const int rr = s_rep[cj];
+            const int k0 = k01 / a.cv.K1, k1 = k01 - k0 * a.cv.K1;
+            bool ok = true;
+            int y0, y1;
+            if (!TRANSPOSED) {
+                y0 = s_c0[rr] * a.cv.s0 - a.cv.p0 + k0;
+                y1 = s_c1[rr] * a.cv.s1 - a.cv.p1 + k1;
+            } else {
+                int t0 = s_c0[rr] + a.cv.p0 - k0, t1 = s_c1[rr] + a.cv.p1 - k1;
+                if (t0 < 0 || t1 < 0 || t0 % a.cv.s0 || t1 % a.cv.s1) ok = false;
+                y0 = t0 / a.cv.s0;
+                y1 = t1 / a.cv.s1;
+            }
+            if (y0 < 0 || y0 >= a.P.n0 || y1 < 0 || y1 >= a.P.n1) ok = false;
+            unsigned long long m = 0;
+            int st = 0;
+            if (ok) {
+                int e;
+                fiber_range(a.p_ptr, (s_b[rr] * a.P.n0 + y0) * a.P.n1 + y1, a.p_rows, st, e);
+                int prev = -1;
+                bool bad = false;
+                for (int e0 = st; e0 < e; e0 += kMaskWalk) {
+                    int v[kMaskWalk];
+#pragma unroll
+                    for (int q = 0; q < kMaskWalk; q++) v[q] = a.p_idx[min(e0 + q, e - 1)];
+#pragma unroll
+                    for (int q = 0; q < kMaskWalk; q++)
+                        if (e0 + q < e) {
+                            if ((unsigned)v[q] >= 64u || v[q] <= prev) bad = true;
+                            else m |= 1ull << v[q];
+                            prev = v[q];
+                        }
+                }
+                if (bad) s_bad = 1;
+            }
+            s_cmask[it] = m;
+            s_cstart[it] = st;
+        }
+        __syncthreads();
+        by_masks = s_bad == 0 && ncols > 0;
+        if (by_masks) {
+            for (int it = tid; it < K01 * R; it += kThreads) {
+                const int rl = it & (R - 1), k01 = it / R;
+                const int cj = s_cj[rl];
+                if (cj < 0) continue;
+                const unsigned long long m = s_cmask[k01 * ncols + cj];
+                if (!m) continue;
+                const int st = s_cstart[k01 * ncols + cj], zz = s_z[rl];
+                for (int k2 = 0; k2 < a.cv.K2; k2++) {
+                    int v;
+                    if (!TRANSPOSED) {
+                        v = zz * a.cv.s2 - a.cv.p2 + k2;
+                    } else {
+                        const int t = zz + a.cv.p2 - k2;
+                        if (t < 0 || t % a.cv.s2) continue;
+                        v = t / a.cv.s2;
+                    }
+                    if ((unsigned)v < 64u && ((m >> v) & 1ull))
+                        s_nbr[rl * KV + k01 * a.cv.K2 + k2] = st + __popcll(m & ((1ull << v) - 1ull));
+                }
+            }
+        }
+    }
+
     // 2. join.  item = (k01, row), consecutive lanes take consecutive rows.  Per pass a
     // thread first issues the two fiber-bound loads of all its items, then the first
     // three S2 coordinates of every fiber, and only then compares; longer fibers finish
     // in a loop.
-    for (int base = 0; base < K01 * R; base += kThreads * kJoinItems) {
+    for (int base = 0; !by_masks && base < K01 * R; base += kThreads * kJoinItems) {
         int ps[kJoinItems], len[kJoinItems], slot[kJoinItems], zz[kJoinItems];
         int raw_e[kJoinItems], raw_s[kJoinItems];
         bool ok[kJoinItems];
@@ -326,9 +433,16 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
             if (len[j] > 0) { int k2 = off + mul * z0[j]; if (k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j]; }
             if (len[j] > 1) { int k2 = off + mul * z1[j]; if (k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j] + 1; }
             if (len[j] > 2) { int k2 = off + mul * z2[j]; if (k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j] + 2; }
-            for (int e = 3; e < len[j]; e++) {
-                int k2 = off + mul * a.p_idx[ps[j] + e];
-                if (k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j] + e;
+            // longer fibers: four entries per round, their loads in flight together
+            for (int e = 3; e < len[j]; e += 4) {
+                int v[4];
+#pragma unroll
+                for (int q = 0; q < 4; q++) v[q] = a.p_idx[ps[j] + min(e + q, len[j] - 1)];
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int k2 = off + mul * v[q];
+                    if (e + q < len[j] && k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j] + e + q;
+                }
             }
         }
     }
@@ -367,114 +481,90 @@ struct OutArgs {
     ConvParams cv;
 };
 
-__device__ unsigned long long column_mask(const OutArgs &a, int b, int o0, int o1, int chunk)
+// Bins of output column (b, o0, o1) inside chunk `chunk` that the input columns k01 = part,
+// part + step, ... reach.
+__device__ unsigned long long column_mask(const OutArgs &a, int b, int o0, int o1, int chunk, int part, int step)
 {
     unsigned long long mask = 0;
-    for (int k0 = 0; k0 < a.cv.K0; k0++) {
+    const int K01 = a.cv.K0 * a.cv.K1;
+    for (int k01 = part; k01 < K01; k01 += step) {
+        const int k0 = k01 / a.cv.K1, k1 = k01 - k0 * a.cv.K1;
         int x0 = o0 * a.cv.s0 - a.cv.p0 + k0;
-        if (x0 < 0 || x0 >= a.S.n0) continue;
-        for (int k1 = 0; k1 < a.cv.K1; k1++) {
-            int x1 = o1 * a.cv.s1 - a.cv.p1 + k1;
-            if (x1 < 0 || x1 >= a.S.n1) continue;
-            int pc = (b * a.S.n0 + x0) * a.S.n1 + x1;
-            int ps, pe;
-            fiber_range(a.z_ptr, pc, a.in_rows, ps, pe);
-            for (int e = ps; e < pe; e++) {
-                int z = a.z_idx[e];
-                for (int k2 = 0; k2 < a.cv.K2; k2++) {
-                    int t = z + a.cv.p2 - k2;
-                    if (t < 0 || t % a.cv.s2) continue;
-                    int o2 = t / a.cv.s2;
-                    if (o2 < a.O.n2 && (o2 >> 6) == chunk) mask |= 1ull << (o2 & 63);
-                }
+        int x1 = o1 * a.cv.s1 - a.cv.p1 + k1;
+        if (x0 < 0 || x0 >= a.S.n0 || x1 < 0 || x1 >= a.S.n1) continue;
+        int pc = (b * a.S.n0 + x0) * a.S.n1 + x1;
+        int ps, pe;
+        fiber_range(a.z_ptr, pc, a.in_rows, ps, pe);
+        for (int e = ps; e < pe; e++) {
+            int z = a.z_idx[e];
+            for (int k2 = 0; k2 < a.cv.K2; k2++) {
+                int t = z + a.cv.p2 - k2;
+                if (t < 0 || t % a.cv.s2) continue;
+                int o2 = t / a.cv.s2;
+                if (o2 < a.O.n2 && (o2 >> 6) == chunk) mask |= 1ull << (o2 & 63);
             }
         }
     }
     return mask;
 }
 
+constexpr int kColLanes = 16;                    // lanes that share one output column
+constexpr int kColsPerBlock = kThreads / kColLanes;
+
+// OR over the 16 lanes of a column group (all 16 are active together).
+__device__ __forceinline__ unsigned long long or_reduce16(unsigned long long m)
+{
+    unsigned lo = (unsigned)m, hi = (unsigned)(m >> 32);
+#pragma unroll
+    for (int off = 1; off < kColLanes; off <<= 1) {
+        lo |= __shfl_xor(lo, off, kWave);
+        hi |= __shfl_xor(hi, off, kWave);
+    }
+    return ((unsigned long long)hi << 32) | lo;
+}
+
+// Per-column counts.  16 lanes share an output column (one input column (k0, k1) each, K0*K1 = 9
+// of them busy for a 3x3x3 kernel), so the fibers that reach a column are walked side by side
+// and small grids still fill the chip.  `masks` (O2 <= 64 only, else null) keeps each column's
+// bin mask for the fill kernel.
 __global__ __launch_bounds__(kThreads) void outcoords_count_kernel(OutArgs a, int32_t *counts,
-                                                                   int32_t *block_sums)
+                                                                   unsigned long long *masks)
 {
-    __shared__ int s_red[kWaves];
     const int ncol = a.B * a.O.n0 * a.O.n1;
-    const int oc = blockIdx.x * kThreads + threadIdx.x;
+    const int part = threadIdx.x % kColLanes;
+    const int oc = blockIdx.x * kColsPerBlock + threadIdx.x / kColLanes;
+    if (oc >= ncol) return; // whole 16-lane groups leave together
+    const int nchunk = (a.O.n2 + 63) >> 6;
+    const int b = oc / (a.O.n0 * a.O.n1);
+    const int rem = oc - b * (a.O.n0 * a.O.n1);
+    const int o0 = rem / a.O.n1, o1 = rem % a.O.n1;
     int cnt = 0;
-    if (oc < ncol) {
-        int b = oc / (a.O.n0 * a.O.n1);
-        int rem = oc - b * (a.O.n0 * a.O.n1);
-        int o0 = rem / a.O.n1, o1 = rem % a.O.n1;
-        int nchunk = (a.O.n2 + 63) >> 6;
-        for (int ch = 0; ch < nchunk; ch++) cnt += __popcll(column_mask(a, b, o0, o1, ch));
-        counts[oc] = cnt;
+    for (int ch = 0; ch < nchunk; ch++) {
+        const unsigned long long m = or_reduce16(column_mask(a, b, o0, o1, ch, part, kColLanes));
+        cnt += __popcll(m);
+        if (masks && part == 0) masks[oc] = m;
     }
-    // block sum
-    int v = cnt;
-    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_down(v, off, kWave);
-    if ((threadIdx.x & (kWave - 1)) == 0) s_red[threadIdx.x / kWave] = v;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int s = 0;
-        for (int w = 0; w < kWaves; w++) s += s_red[w];
-        block_sums[blockIdx.x] = s;
-    }
+    if (part == 0) counts[oc] = cnt;
 }
 
-// Exclusive scan of block_sums[n] in place by one block; total -> *total.
-__global__ __launch_bounds__(1024) void scan_block_sums_kernel(int32_t *block_sums, int n, int32_t *total)
-{
-    __shared__ int s_buf[1024];
-    __shared__ int s_carry;
-    if (threadIdx.x == 0) s_carry = 0;
-    __syncthreads();
-    for (int base = 0; base < n; base += 1024) {
-        int i = base + threadIdx.x;
-        int v = (i < n) ? block_sums[i] : 0;
-        s_buf[threadIdx.x] = v;
-        __syncthreads();
-        for (int off = 1; off < 1024; off <<= 1) {
-            int t = (threadIdx.x >= off) ? s_buf[threadIdx.x - off] : 0;
-            __syncthreads();
-            s_buf[threadIdx.x] += t;
-            __syncthreads();
-        }
-        int incl = s_buf[threadIdx.x];
-        int carry = s_carry;
-        if (i < n) block_sums[i] = carry + incl - v;
-        __syncthreads();
-        if (threadIdx.x == 1023) s_carry = carry + incl;
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) *total = s_carry;
-}
+__global__ void copy_last_kernel(const int32_t *v, int n, int32_t *out) { *out = n > 0 ? v[n - 1] : 0; }
 
-__global__ __launch_bounds__(kThreads) void outcoords_fill_kernel(OutArgs a, const int32_t *block_offs,
-                                                                  int32_t *oz_ptr, int32_t *oz_idx,
-                                                                  int out_rows)
+// oz_ptr holds the inclusive scan of the counts; one thread writes the bins of one column.
+__global__ __launch_bounds__(kThreads) void outcoords_fill_kernel(OutArgs a, const int32_t *oz_ptr, int32_t *oz_idx,
+                                                                  int out_rows, const unsigned long long *masks)
 {
-    __shared__ int s_buf[kThreads];
     const int ncol = a.B * a.O.n0 * a.O.n1;
     const int oc = blockIdx.x * kThreads + threadIdx.x;
-    int cnt = (oc < ncol) ? oz_ptr[oc] : 0; // per-column count left by the count kernel
-    s_buf[threadIdx.x] = cnt;
-    __syncthreads();
-    for (int off = 1; off < kThreads; off <<= 1) {
-        int t = (threadIdx.x >= off) ? s_buf[threadIdx.x - off] : 0;
-        __syncthreads();
-        s_buf[threadIdx.x] += t;
-        __syncthreads();
-    }
     if (oc >= ncol) return;
-    int incl = block_offs[blockIdx.x] + s_buf[threadIdx.x];
-    oz_ptr[oc] = incl;
-    if (cnt == 0) return;
-    int pos = incl - cnt;
+    int pos = oc ? oz_ptr[oc - 1] : 0;
+    const int end = oz_ptr[oc];
+    if (end <= pos) return;
     int b = oc / (a.O.n0 * a.O.n1);
     int rem = oc - b * (a.O.n0 * a.O.n1);
     int o0 = rem / a.O.n1, o1 = rem % a.O.n1;
     int nchunk = (a.O.n2 + 63) >> 6;
     for (int ch = 0; ch < nchunk; ch++) {
-        unsigned long long m = column_mask(a, b, o0, o1, ch);
+        unsigned long long m = masks ? masks[oc] : column_mask(a, b, o0, o1, ch, 0, 1);
         while (m) {
             int bit = __ffsll((long long)m) - 1;
             if (pos < out_rows) oz_idx[pos] = ch * 64 + bit;
@@ -594,7 +684,7 @@ void sph_set_error(const char *fmt, ...)
 }
 
 SPH_EXPORT const char *sph_last_error(void) { return g_err; }
-SPH_EXPORT int sph_abi_version(void) { return 1; }
+SPH_EXPORT int sph_abi_version(void) { return 2; }
 SPH_EXPORT int sph_book_tiles(int rows) { return rows <= 0 ? 0 : sph_div_up(rows, R); }
 SPH_EXPORT int sph_book_cap(int KV) { return KV * (R / SPH_GROUP); }
 
@@ -651,7 +741,12 @@ static int rules_build(const char *who, const int32_t *z_idx, const int32_t *z_p
         a.pack.total = 0;
     }
     if (a.tile_blocks + pack_blocks == 0) return SPH_OK;
-    const size_t lds = (size_t)R * KV * sizeof(int32_t);
+    size_t lds = (size_t)R * KV * sizeof(int32_t);
+    // masks pay when a fiber of the gathered side serves several rows: four entries on average
+    const long p_cols = (long)a.B * a.P.n0 * a.P.n1;
+    const size_t lds_masks = (size_t)kMaskCols * (g->K[0] * g->K[1]) * (sizeof(unsigned long long) + sizeof(int32_t));
+    a.long_fibers = a.P.n2 <= 64 && (long)a.p_rows >= 4 * p_cols && lds + lds_masks <= 64 * 1024;
+    if (a.long_fibers) lds += lds_masks;
     hipStream_t st = (hipStream_t)stream;
     if (!transposed)
         hipLaunchKernelGGL(build_book_kernel<false>, dim3(a.tile_blocks + pack_blocks), dim3(kThreads), lds, st, a);
@@ -687,6 +782,34 @@ SPH_EXPORT int sph_outcoords_blocks(const sph_geom *g)
     return sph_div_up(g->B * g->O[0] * g->O[1], kThreads);
 }
 
+static size_t outcoords_scan_bytes(long ncol)
+{
+    size_t bytes = 0;
+    hipError_t e = rocprim::inclusive_scan(nullptr, bytes, (int32_t *)nullptr, (int32_t *)nullptr, (size_t)(ncol > 0 ? ncol : 1),
+                                           rocprim::plus<int32_t>(), (hipStream_t)0);
+    return e == hipSuccess ? bytes + 8 : 0;
+}
+
+// int32 entries of the scratch the two calls share: the scan's temporary storage and, when a
+// column's bins fit one 64-bit mask, the masks (8-byte aligned behind it)
+SPH_EXPORT int sph_outcoords_scratch_ints(const sph_geom *g)
+{
+    SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_scratch_ints: bad geometry");
+    const long ncol = (long)g->B * g->O[0] * g->O[1];
+    const size_t scan = outcoords_scan_bytes(ncol);
+    SPH_REQUIRE(scan != 0, SPH_ERR_LAUNCH, "sph_outcoords_scratch_ints: temporary storage query failed");
+    const long n = (long)((scan + 7) / 8 * 2) + (g->O[2] <= 64 ? 2 * ncol : 0);
+    SPH_REQUIRE(n < 2147483647L, SPH_ERR_UNSUPPORTED, "sph_outcoords_scratch_ints: grid too large");
+    return (int)n;
+}
+
+static unsigned long long *outcoords_masks(const sph_geom *g, int32_t *scratch)
+{
+    if (g->O[2] > 64) return nullptr;
+    const long ncol = (long)g->B * g->O[0] * g->O[1];
+    return (unsigned long long *)(scratch + (outcoords_scan_bytes(ncol) + 7) / 8 * 2);
+}
+
 static OutArgs out_args(const int32_t *z_idx, const int32_t *z_ptr, int in_rows, const sph_geom *g)
 {
     OutArgs a;
@@ -698,32 +821,41 @@ static OutArgs out_args(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
 }
 
 SPH_EXPORT int sph_outcoords_count(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
-                                   const sph_geom *g, int32_t *oz_ptr, int32_t *block_sums,
+                                   const sph_geom *g, int32_t *oz_ptr, int32_t *scratch,
                                    int32_t *total_dev, void *stream)
 {
     SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_count: bad geometry");
-    SPH_REQUIRE(z_ptr && oz_ptr && block_sums && total_dev && in_rows >= 0 && (in_rows == 0 || z_idx),
+    SPH_REQUIRE(z_ptr && oz_ptr && scratch && total_dev && in_rows >= 0 && (in_rows == 0 || z_idx),
                 SPH_ERR_ARG, "sph_outcoords_count: null argument");
+    SPH_REQUIRE((uintptr_t)scratch % 8 == 0, SPH_ERR_ARG, "sph_outcoords_count: scratch must be 8-byte aligned");
     hipStream_t st = (hipStream_t)stream;
-    const int nb = sph_outcoords_blocks(g);
-    hipLaunchKernelGGL(outcoords_count_kernel, dim3(nb), dim3(kThreads), 0, st,
-                       out_args(z_idx, z_ptr, in_rows, g), oz_ptr, block_sums);
+    const int ncol = g->B * g->O[0] * g->O[1];
+    hipLaunchKernelGGL(outcoords_count_kernel, dim3(sph_div_up(ncol, kColsPerBlock)), dim3(kThreads), 0, st,
+                       out_args(z_idx, z_ptr, in_rows, g), oz_ptr, outcoords_masks(g, scratch));
     int rc = sph_check_launch("sph_outcoords_count");
     if (rc) return rc;
-    hipLaunchKernelGGL(scan_block_sums_kernel, dim3(1), dim3(1024), 0, st, block_sums, nb, total_dev);
-    return sph_check_launch("sph_outcoords_count(scan)");
+    size_t bytes = outcoords_scan_bytes(ncol);
+    SPH_REQUIRE(bytes != 0, SPH_ERR_LAUNCH, "sph_outcoords_count: temporary storage query failed");
+    hipError_t e = rocprim::inclusive_scan((void *)scratch, bytes, oz_ptr, oz_ptr, (size_t)ncol, rocprim::plus<int32_t>(), st);
+    if (e != hipSuccess) {
+        sph_set_error("sph_outcoords_count: scan: %s", hipGetErrorString(e));
+        return SPH_ERR_LAUNCH;
+    }
+    hipLaunchKernelGGL(copy_last_kernel, dim3(1), dim3(1), 0, st, (const int32_t *)oz_ptr, ncol, total_dev);
+    return sph_check_launch("sph_outcoords_count(total)");
 }
 
 SPH_EXPORT int sph_outcoords_fill(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
-                                  const sph_geom *g, const int32_t *block_sums, int32_t *oz_ptr,
+                                  const sph_geom *g, const int32_t *scratch, int32_t *oz_ptr,
                                   int32_t *oz_idx, int out_rows, void *stream)
 {
     SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_fill: bad geometry");
-    SPH_REQUIRE(z_ptr && oz_ptr && block_sums && out_rows >= 0 && (out_rows == 0 || oz_idx) &&
+    SPH_REQUIRE(z_ptr && oz_ptr && scratch && out_rows >= 0 && (out_rows == 0 || oz_idx) &&
                     (in_rows == 0 || z_idx), SPH_ERR_ARG, "sph_outcoords_fill: null argument");
     const int nb = sph_outcoords_blocks(g);
     hipLaunchKernelGGL(outcoords_fill_kernel, dim3(nb), dim3(kThreads), 0, (hipStream_t)stream,
-                       out_args(z_idx, z_ptr, in_rows, g), block_sums, oz_ptr, oz_idx, out_rows);
+                       out_args(z_idx, z_ptr, in_rows, g), (const int32_t *)oz_ptr, oz_idx, out_rows,
+                       (const unsigned long long *)outcoords_masks(g, (int32_t *)scratch));
     return sph_check_launch("sph_outcoords_fill");
 }
 

@@ -159,9 +159,10 @@ class RuleBook:
         g = L.make_geom(batch, in_shape, out_shape, kernel, stride, padding, dilation)
         if min(int(v) for v in out_shape) <= 0:
             raise L.SphconvError("empty output grid %s" % (list(out_shape),))
-        nblk = lib.sph_outcoords_blocks(C.byref(g))
+        nblk = lib.sph_outcoords_scratch_ints(C.byref(g))
         if nblk < 0:
             L.check(nblk)
+        nblk += nblk & 1                                      # the total sits behind an even count
         oz_ptr = torch.empty((int(batch), int(out_shape[0]), int(out_shape[1])), dtype=torch.int32, device=dev)
         scratch = torch.empty(nblk + 1, dtype=torch.int32, device=dev)
         total = scratch[nblk:]

@@ -214,21 +214,22 @@ def test_fused_eval_tail_equals_separate_modules():
     # the affine map kept on a BatchNorm module follows in-place changes of its tensors
     net.fuse_eval = True
     with torch.no_grad():
+        w0, m0 = net[1].weight.clone(), net[1].running_mean.clone()
         net[1].weight.mul_(-1.5)
         net[1].running_mean.add_(0.25)
         fused2 = net(sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx)))
         net.fuse_eval = False
         plain2 = net(sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx)))
-        net[1].weight.div_(-1.5)
-        net[1].running_mean.sub_(0.25)
+        net[1].weight.copy_(w0)
+        net[1].running_mean.copy_(m0)
     assert not torch.allclose(plain2.feature.float(), plain.feature.float(), rtol=2e-2, atol=2e-2)
-    torch.testing.assert_close(fused2.feature.float(), plain2.feature.float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(fused2.feature.float(), plain2.feature.float(), rtol=3e-2, atol=5e-2)
     # with gradients enabled nothing is fused (autograd needs the separate modules)
     net.fuse_eval = True
     x3 = sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx))
     y3 = net(x3)
     assert y3.feature.requires_grad
-    torch.testing.assert_close(y3.feature.detach().float(), plain.feature.float(), rtol=2e-3, atol=2e-3)
+    assert torch.equal(y3.feature.detach(), plain.feature)
 
 
 def test_config4_encoder_full_size_layer_by_layer():

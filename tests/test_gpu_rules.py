@@ -217,3 +217,29 @@ def test_init_tensor_sizes(B, shape, n):
     g = rng.standard_normal(f.shape).astype(np.float32)
     back = ext.init_tensor_backward(G.t(g), G.t(perm)).cpu().numpy()
     assert np.array_equal(back, g[perm])
+
+
+def test_unsorted_long_fibers_take_the_general_join():
+    """Long fibers are joined through per-column bin masks, which needs them in ascending S2 order
+    (as init_tensor and the strided rule generation emit them); a tensor whose fibers are in another
+    order (legal in the reference: tensor.cu:61-65 leaves the order to the atomics) must give the
+    same pairs through the general join."""
+    rng = np.random.default_rng(11)
+    B, shape = 2, [6, 9, 16]
+    occ = rng.random((B, *shape)) < 0.6
+    idx = np.argwhere(occ).astype(np.int32)
+    _, z_idx, z_ptr, _ = H.csr_from_indices(idx, B, shape)
+    assert z_idx.shape[0] >= 4 * B * shape[0] * shape[1]
+    ends = z_ptr.reshape(-1)
+    starts = np.concatenate([[0], ends[:-1]])
+    z_rev = z_idx.copy()
+    for s, e in zip(starts, ends):
+        z_rev[s:e] = z_idx[s:e][::-1]
+    assert not np.array_equal(z_rev, z_idx)
+    for zi in (z_idx, z_rev):
+        book = RuleBook.build_subm(G.t(zi), G.t(z_ptr), B, shape, [3, 3, 3])
+        _, _, rules, rule_size, dropped = O.get_rules_subm(zi, z_ptr, B, shape, shape, [3, 3, 3], [1, 1, 1], [1, 1, 1],
+                                                           (1, 1, 1), (2, 2), n_max=256)
+        assert dropped == 0
+        assert np.array_equal(G.book_triples(book.fwd), G.oracle_triples(rules, rule_size))
+        assert np.array_equal(G.book_triples(book.transposed()), G.oracle_triples(rules, rule_size, swap=True))
