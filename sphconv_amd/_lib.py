@@ -41,6 +41,7 @@ class Epilogue(C.Structure):
 
 
 _lib = None
+ABI_VERSION = 2       # sph_abi_version() of the library these signatures describe
 
 _I, _P, _L, _Z = C.c_int, C.c_void_p, C.c_long, C.c_size_t
 _SIGNATURES = {
@@ -92,6 +93,9 @@ def lib():
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
+        if handle.sph_abi_version() != ABI_VERSION:
+            raise SphconvError("%s has ABI version %d, this package needs %d: rebuild it (make -C sphconv_amd/csrc)"
+                               % (LIB_PATH, handle.sph_abi_version(), ABI_VERSION))
         _lib = handle
     return _lib
 
