@@ -48,6 +48,9 @@ def parse():
     ap.add_argument("--encoder", action="store_true",
                     help="also time configuration 4 (four-stage encoder, batch 4, fp16, rules regenerated every "
                          "pass) end to end; reported under 'encoder_stack', not part of 'value'")
+    ap.add_argument("--callers", action="store_true",
+                    help="also time the callers either side of the path (init_tensor, to_dense, xyz2RangeVoxel, "
+                         "points_to_voxel_v2 + mean VFE) with HIP events; reported under 'callers'")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 256 MiB device-to-device copies (a kernel of known HBM traffic, "
@@ -144,6 +147,63 @@ def encoder_stack_ms(torch, seed, iters):
             res["ms_per_scan"] = res[key] / B
             res["voxels_out"] = int(y.feature.shape[0])
     return res
+
+
+def callers_ms(torch, d, seed, iters):
+    """The functions either side of the convolution, each timed alone (HIP events around `iters` calls, so a
+    call's own device->host read is part of its time).  `bytes` = what the call must read and write."""
+    import numpy as np
+    from sphconv_amd import sphconv_cuda as ext
+    from sphconv_amd.data import xyz2RangeVoxel
+    from sphconv_amd.synth import make_config
+    from sphconv_amd.vfe import SimpleVoxel
+    from sphconv_amd.voxelize import VoxelGeneratorV3
+    dev = "cuda:0"
+    rng = np.random.default_rng(seed)
+    out = {}
+
+    def timed(name, fn, nbytes, note):
+        ms = event_ms(fn, iters, torch)
+        out[name] = {"ms": ms, "bytes": nbytes, "GBps": nbytes / (ms * 1e-3) / 1e9, "workload": note}
+
+    # COO -> compressed layout of the headline scan (rows in random order), 64 fp16 channels
+    n, (S0, S1, S2), B = int(d["z_idx"].shape[0]), d["spatial_shape"], d["batch"]
+    perm = rng.permutation(n)
+    idx = torch.tensor(d["indices"][perm], device=dev)
+    feat = torch.tensor(rng.standard_normal((n, 64)), dtype=torch.float32, device=dev).half()
+    timed("init_tensor", lambda: ext.init_tensor(feat, idx, B, [S0, S1, S2]),
+          n * (16 + 4 + 4 + 2 * 128) + 4 * B * S0 * S1, "%d voxels, grid %dx%dx%d, 64 fp16 channels" % (n, S0, S1, S2))
+    # densify and its backward at configuration 1 (16 fp32 channels)
+    c1 = make_config(1, seed=seed)
+    n1, (T0, T1, T2) = int(c1["z_idx"].shape[0]), c1["spatial_shape"]
+    zi1, zp1 = torch.tensor(c1["z_idx"], device=dev), torch.tensor(c1["z_ptr"], device=dev)
+    f1 = torch.tensor(rng.standard_normal((n1, 16)), dtype=torch.float32, device=dev)
+    dense = torch.empty((1, T0, T1, T2, 16), dtype=torch.float32, device=dev)
+    timed("to_dense", lambda: ext.to_dense(f1, zi1, zp1, T2, dense), n1 * (64 + 64 + 4) + 4 * T0 * T1,
+          "%d rows of 16 fp32 written into their cells of a zeroed dense %dx%dx%dx16 tensor" % (n1, T0, T1, T2))
+    timed("to_dense_backward", lambda: ext.to_dense_backward(dense, zi1, zp1), n1 * (128 + 4) + 4 * T0 * T1,
+          "gather of %d rows of 16 fp32 from the dense gradient" % n1)
+    # one synthetic HDL-64-like sweep of the front sector: 122 880 points (x, y, z, reflectance)
+    m = 64 * 1920
+    theta = np.deg2rad(rng.uniform(87.5, 103.4, m))
+    phi = np.deg2rad(rng.uniform(-45, 45, m))
+    r = rng.uniform(6.0, 70.0, m)
+    pts = np.stack([r * np.sin(theta) * np.cos(phi), r * np.sin(theta) * np.sin(phi), r * np.cos(theta),
+                    rng.random(m)], 1).astype(np.float32)
+    pts_d = torch.tensor(pts, device=dev)
+    timed("xyz2RangeVoxel", lambda: xyz2RangeVoxel(pts_d), m * 16 + 64 * 512 * (16 + 4 + 4 + 4),
+          "%d points -> range image 64x512, 512 depth bins" % m)
+    gen = VoxelGeneratorV3(None, [6, -40, -3, 70.4, 40, 1], [6, -45, 87.5, 70.4, 45, 100], 2, 24000, [512, 512, 64],
+                           coord_system="spherical")
+    vfe = SimpleVoxel(4)
+
+    def voxelise():
+        res = gen.generate(pts_d)
+        return vfe(res["voxels"], res["num_points_per_voxel"], res["coordinates"])
+
+    timed("points_to_voxel_v2+SimpleVoxel", voxelise, m * (16 + 8 + 8) + 24000 * (2 * 16 + 8 + 12 + 4 + 16),
+          "%d points -> at most 24000 voxels of 2 points on a 512x512x64 spherical grid, mean VFE" % m)
+    return out
 
 
 def main():
@@ -276,6 +336,8 @@ def main():
                     "conv_TFLOPs": conv_flops / (conv_ms * 1e-3) / 1e12, **extra},
         "roofline": roofline,
     }
+    if args.callers:
+        result["callers"] = callers_ms(torch, d, args.seed, 50)
     if args.encoder:
         result["encoder_stack"] = encoder_stack_ms(torch, args.seed, 20)
     if not args.no_cpu_baseline:
