@@ -173,7 +173,7 @@ __global__ void coo_scatter_kernel(const int32_t *idx, int n, int S0, int S1, co
     seg_row[pos] = i;
 }
 
-__global__ void coo_rank_kernel(const int32_t *idx, int n, int S0, int S1, const int32_t *z_ptr, const int32_t *slot,
+__global__ void coo_rank_kernel(const int32_t *idx, int n, int S0, int S1, int S2, const int32_t *z_ptr, const int32_t *slot,
                                 const int32_t *seg_z, const int32_t *seg_row, int32_t *z_idx, int32_t *permutation,
                                 int32_t *status)
 {
@@ -183,8 +183,12 @@ __global__ void coo_rank_kernel(const int32_t *idx, int n, int S0, int S1, const
     const int4 c = ((const int4 *)idx)[i];
     const int col = (c.x * S0 + c.y) * S1 + c.z;
     const int start = col ? z_ptr[col - 1] : 0;
-    const int end = min(z_ptr[col], n);
+    int end = min(z_ptr[col], n);
     int rank = 0, dup = 0;
+    if (end - start > S2) { // more rows than bins: duplicates for sure; keep the walk bounded
+        dup = 1;
+        end = start + S2;
+    }
     for (int j = start; j < end; j++) {
         const int z = seg_z[j];
         rank += z < c.w;
@@ -236,7 +240,7 @@ static int init_tensor_by_rank(const int32_t *indices, int n, int B, int S0, int
     }
     hipLaunchKernelGGL(coo_scatter_kernel, grid, block, 0, st, indices, n, S0, S1, (const int32_t *)z_ptr,
                        (const int32_t *)slot, seg_z, seg_row);
-    hipLaunchKernelGGL(coo_rank_kernel, grid, block, 0, st, indices, n, S0, S1, (const int32_t *)z_ptr, (const int32_t *)slot,
+    hipLaunchKernelGGL(coo_rank_kernel, grid, block, 0, st, indices, n, S0, S1, S2, (const int32_t *)z_ptr, (const int32_t *)slot,
                        (const int32_t *)seg_z, (const int32_t *)seg_row, z_idx, permutation, status);
     return sph_check_launch("sph_init_tensor(rank)");
 }

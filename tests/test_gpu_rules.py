@@ -186,6 +186,10 @@ def test_extension_functions_match_reference_signatures():
     bad = idx.copy(); bad[0, 3] = 99
     with pytest.raises(ValueError):
         ext.init_tensor(G.t(feat), G.t(bad), 2, [8, 9, 9])
+    # 50 000 copies of one coordinate: reported as duplicates without walking the column once per copy
+    many = np.repeat(idx[:1], 50000, axis=0)
+    with pytest.raises(ValueError, match="duplicate"):
+        ext.init_tensor(G.t(np.zeros((50000, 2), np.float32)), G.t(many), 2, [8, 9, 9])
 
 
 @pytest.mark.parametrize("B,shape,n", [(1, (64, 512, 32), 40000), (3, (7, 5, 3), 50), (2, (2048, 2048, 1024), 3000),
