@@ -85,6 +85,12 @@ typedef struct sph_book {
     int32_t *grp_owner;
     int32_t rows; /* rows on the stationary side */
     int32_t KV;
+    /* Optional second form of the same pairs, by stationary row: [NT][KV][SPH_TILE_ROWS],
+     * gathered row of (tile, offset, row of the tile) or -1.  When not null, sph_rules_build*
+     * and sph_rules_from_padded fill it too, and sph_conv_apply walks it instead of the groups
+     * (every offset of every block of 16 rows costs one step, whatever it holds: the faster
+     * way from about six pairs per row upwards).  Null: not kept. */
+    int32_t *tile_nbr;
 } sph_book;
 
 const char *sph_last_error(void);

@@ -33,7 +33,7 @@ class Geom(C.Structure):
 class Book(C.Structure):
     _fields_ = [("tile_ngrp", C.c_void_p), ("tile_koff", C.c_void_p), ("grp_k", C.c_void_p),
                 ("grp_gather", C.c_void_p), ("grp_owner", C.c_void_p), ("rows", C.c_int32),
-                ("KV", C.c_int32)]
+                ("KV", C.c_int32), ("tile_nbr", C.c_void_p)]
 
 
 class Epilogue(C.Structure):
@@ -41,7 +41,7 @@ class Epilogue(C.Structure):
 
 
 _lib = None
-ABI_VERSION = 2       # sph_abi_version() of the library these signatures describe
+ABI_VERSION = 3       # sph_abi_version() of the library these signatures describe
 
 _I, _P, _L, _Z = C.c_int, C.c_void_p, C.c_long, C.c_size_t
 _SIGNATURES = {

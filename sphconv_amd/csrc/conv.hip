@@ -496,6 +496,151 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
 }
 
 // ---------------------------------------------------------------------------
+// Walk by stationary row (book.tile_nbr): for dense neighbourhoods.
+//
+// The grouped kernel above pays per group of 16 pairs (weight fragments through the L1,
+// an LDS read-modify-write of the owners' accumulators), which is the right price when a
+// row has two or three pairs.  From about six pairs per row upwards it is cheaper to take
+// every (offset, block of 16 consecutive rows) in turn, whatever it holds: the 16 gathered
+// rows (zeros where a row has no pair at this offset) times the offset's weight, added to
+// accumulators that never leave the registers (8 blocks x 64 columns = 128 per lane).
+// 27 weight loads per tile instead of one per group, no LDS, no owner indirection; the
+// price is one MFMA step per (offset, block) even when it is nearly empty.
+// One wave per tile and 64 output columns; rows are requested half a tile (4 blocks)
+// ahead of their use.
+// ---------------------------------------------------------------------------
+template <sph_dtype DT, int NS, int CT, bool MASKED>
+__global__ __launch_bounds__(128) void conv_rows_kernel(ConvArgs a, int nwtot)
+{
+    typedef typename Traits<DT>::elem elem;
+    typedef typename Traits<DT>::acc4 acc4;
+    constexpr int HB = R / SPH_GROUP / 2; // blocks of 16 rows per half tile
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int tile = sph_xcd_tile(blockIdx.x, (a.book.rows + R - 1) / R);
+    const int r0 = tile * R;
+    if (r0 >= a.book.rows) return;
+    const int nrows = min(R, a.book.rows - r0);
+    const int col0 = wave * CT * 16;
+    const int KV = a.book.KV;
+    const int32_t *nb = a.book.tile_nbr + (long)tile * KV * R;
+    const char *wlane = a.wp + ((long)(wave * CT)) * (kWave * 16) + lane * 16;
+    const long wstep = (long)nwtot * (kWave * 16);
+
+    auto load_idx = [&](int k, int &lo, int &hi) { // rows 0..63 and 64..127 of offset k (clamped: always readable)
+        const int kk = min(k, KV - 1);
+        lo = nb[kk * R + lane];
+        hi = nb[kk * R + kWave + lane];
+    };
+    auto check_idx = [&](int &v) { v = (unsigned)v < (unsigned)a.feat_rows ? v : -1; };
+    auto issue_rows = [&](int sel, int4v (&fa)[HB][NS], int (&rows)[HB]) {
+#pragma unroll
+        for (int j = 0; j < HB; j++) {
+            rows[j] = __shfl(sel, j * SPH_GROUP + (lane & 15), kWave);
+            const char *row = a.feat + (long)max(rows[j], 0) * a.row_bytes;
+#pragma unroll
+            for (int st = 0; st < NS; st++) {
+                const int off = st * 64 + (lane >> 4) * 16;
+                fa[j][st] = *(const int4v *)(row + (off < a.row_bytes ? off : 0));
+            }
+        }
+    };
+    auto load_w = [&](int k, int4v (&fw)[NS][CT]) {
+        const char *wk = wlane + (long)k * NS * wstep;
+#pragma unroll
+        for (int st = 0; st < NS; st++)
+#pragma unroll
+            for (int c = 0; c < CT; c++) fw[st][c] = *(const int4v *)(wk + st * wstep + (long)c * (kWave * 16));
+    };
+    auto compute = [&](const int4v (&fw)[NS][CT], const int4v (&fa)[HB][NS], const int (&rows)[HB], acc4 (&ac)[HB][CT]) {
+#pragma unroll
+        for (int j = 0; j < HB; j++)
+#pragma unroll
+            for (int st = 0; st < NS; st++) {
+                bool live = rows[j] >= 0;
+                if constexpr (MASKED) live = live && (st * 64 + (lane >> 4) * 16 < a.row_bytes);
+                const int4v x = live ? fa[j][st] : int4v{0, 0, 0, 0};
+#pragma unroll
+                for (int c = 0; c < CT; c++) ac[j][c] = mfma_step<DT>(fw[st][c], x, ac[j][c]);
+            }
+    };
+
+    acc4 acc_lo[HB][CT], acc_hi[HB][CT];
+#pragma unroll
+    for (int j = 0; j < HB; j++)
+#pragma unroll
+        for (int c = 0; c < CT; c++) acc_lo[j][c] = acc_hi[j][c] = acc4{0, 0, 0, 0};
+
+    int lo, hi, lo_n, hi_n;
+    load_idx(0, lo, hi);
+    load_idx(1, lo_n, hi_n);
+    check_idx(lo);
+    check_idx(hi);
+    int4v fa0[HB][NS], fa1[HB][NS];
+    int rw0[HB], rw1[HB];
+    issue_rows(lo, fa0, rw0);
+    for (int k = 0; k < KV; k++) {
+        int4v fw[NS][CT];
+        load_w(k, fw);
+        issue_rows(hi, fa1, rw1);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(fw, fa0, rw0, acc_lo);
+        __builtin_amdgcn_sched_barrier(0);
+        lo = lo_n;
+        hi = hi_n;
+        check_idx(lo);
+        check_idx(hi);
+        load_idx(k + 2, lo_n, hi_n);
+        issue_rows(lo, fa0, rw0); // first half of the next offset (of the last one again after the last: unused)
+        __builtin_amdgcn_sched_barrier(0);
+        compute(fw, fa1, rw1, acc_hi);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // epilogue: a lane holds four consecutive columns of one row per block and column tile
+    const bool plain = DT != SPH_I8 && !a.scale && !a.shift && !a.relu;
+    const bool relu = DT != SPH_I8 && a.relu;
+    float sc[CT][4], sh[CT][4];
+#pragma unroll
+    for (int c = 0; c < CT; c++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int col = min(col0 + c * 16 + (lane >> 4) * 4 + j, a.ndim - 1);
+            sc[c][j] = a.scale ? a.scale[col] : 1.f;
+            sh[c][j] = (DT != SPH_I8 && a.shift) ? a.shift[col] : 0.f;
+        }
+    elem *out = (elem *)a.out + (long)r0 * a.ndim;
+    auto store_block = [&](int b, const acc4 (&ac)[CT]) {
+        const int row = b * SPH_GROUP + (lane & 15);
+        if (row >= nrows) return;
+#pragma unroll
+        for (int c = 0; c < CT; c++) {
+            const int col = col0 + c * 16 + (lane >> 4) * 4;
+            if (col >= a.ndim) continue;
+            union { elem e[4]; uint32_t w[sizeof(elem)]; } u;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float v = DT == SPH_I8 ? (float)(int)ac[c][j] : (float)ac[c][j];
+                if (!plain) {
+                    v = v * sc[c][j] + sh[c][j];
+                    if (relu) v = v > 0.f ? v : 0.f;
+                }
+                u.e[j] = to_elem<DT>(v);
+            }
+            uint32_t *dst = (uint32_t *)(out + (long)row * a.ndim + col);
+#pragma unroll
+            for (int q = 0; q < (int)sizeof(elem); q++) dst[q] = u.w[q];
+        }
+    };
+#pragma unroll
+    for (int j = 0; j < HB; j++) store_block(j, acc_lo[j]);
+#pragma unroll
+    for (int j = 0; j < HB; j++) store_block(HB + j, acc_hi[j]);
+}
+
+// ---------------------------------------------------------------------------
 // wgrad
 // ---------------------------------------------------------------------------
 struct WgradArgs {
@@ -980,9 +1125,38 @@ int launch_conv_wave_ct(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st
     }
 }
 
+template <sph_dtype DT, int NS, int CT>
+int launch_conv_rows(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
+{
+    const int waves = (nwtot + CT - 1) / CT;
+    if (a.row_bytes < NS * 64)
+        hipLaunchKernelGGL((conv_rows_kernel<DT, NS, CT, true>), dim3(sph_xcd_grid(ntiles)), dim3(waves * kWave), 0, st, a, nwtot);
+    else
+        hipLaunchKernelGGL((conv_rows_kernel<DT, NS, CT, false>), dim3(sph_xcd_grid(ntiles)), dim3(waves * kWave), 0, st, a, nwtot);
+    return sph_check_launch("sph_conv_apply");
+}
+
+template <sph_dtype DT, int NS>
+int launch_conv_rows_ct(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
+{
+    switch (nwtot) {
+    case 1: return launch_conv_rows<DT, NS, 1>(a, nwtot, ntiles, st);
+    case 2: return launch_conv_rows<DT, NS, 2>(a, nwtot, ntiles, st);
+    default: return launch_conv_rows<DT, NS, 4>(a, nwtot, ntiles, st);
+    }
+}
+
 template <sph_dtype DT, int NW>
 int launch_conv(const ConvArgs &a, int ntiles, hipStream_t st)
 {
+    if (a.aligned_in && a.aligned_out && a.feat_rows > 0 && a.book.tile_nbr) {
+        switch (a.nsteps) {
+        case 1: return launch_conv_rows_ct<DT, 1>(a, NW, ntiles, st);
+        case 2: return launch_conv_rows_ct<DT, 2>(a, NW, ntiles, st);
+        case 4: return launch_conv_rows_ct<DT, 4>(a, NW, ntiles, st);
+        default: break;
+        }
+    }
     if (a.aligned_in && a.feat_rows > 0) {
         switch (a.nsteps) {
         case 1: return launch_conv_wave_ct<DT, 1>(a, NW, ntiles, st);

@@ -123,6 +123,14 @@ __device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int t
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
 
+    if (book.tile_nbr) { // the same pairs by stationary row: [k][row of the tile], coalesced
+        int32_t *dst = book.tile_nbr + (long)tile * KV * R;
+        for (int i = tid; i < KV * R; i += kThreads) {
+            const int k = i / R, r = i - k * R;
+            dst[i] = r < nrows ? nbr[r * KV + k] : -1;
+        }
+    }
+
     for (int k = wave; k < KV; k += kWaves) {
         int r_lo = lane, r_hi = kWave + lane;
         unsigned long long m0 = __ballot(r_lo < nrows && nbr[r_lo * KV + k] >= 0);
@@ -684,7 +692,7 @@ void sph_set_error(const char *fmt, ...)
 }
 
 SPH_EXPORT const char *sph_last_error(void) { return g_err; }
-SPH_EXPORT int sph_abi_version(void) { return 2; }
+SPH_EXPORT int sph_abi_version(void) { return 3; }
 SPH_EXPORT int sph_book_tiles(int rows) { return rows <= 0 ? 0 : sph_div_up(rows, R); }
 SPH_EXPORT int sph_book_cap(int KV) { return KV * (R / SPH_GROUP); }
 

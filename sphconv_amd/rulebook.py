@@ -19,16 +19,19 @@ class _Buffers:
     (a single caching-allocator call per book); the named tensors are views made on
     first access."""
 
-    _FIELDS = ("tile_ngrp", "tile_koff", "grp_k", "grp_gather", "grp_owner")
+    _FIELDS = ("tile_ngrp", "tile_koff", "grp_k", "grp_gather", "grp_owner", "tile_nbr")
 
-    def __init__(self, rows: int, kv: int, device):
+    def __init__(self, rows: int, kv: int, device, by_row: bool = False):
+        """``by_row`` also keeps the pairs by stationary row (``tile_nbr`` [NT,KV,128]), the form the
+        convolution walks when neighbourhoods are dense."""
         lib = L.lib()
         self.rows, self.kv = int(rows), int(kv)
         self.ntiles = lib.sph_book_tiles(self.rows)
         self.cap = lib.sph_book_cap(self.kv)
+        self.by_row = bool(by_row)
         nt = max(self.ntiles, 1)
         sizes = (nt * 4, nt * (self.kv + 1) * 2, nt * self.cap * 4, nt * self.cap * L.GROUP * 4,
-                 nt * self.cap * L.GROUP * 4)
+                 nt * self.cap * L.GROUP * 4, nt * self.kv * L.TILE_ROWS * 4 if by_row else 0)
         self._off = []
         total = 0
         for sz in sizes:
@@ -37,7 +40,8 @@ class _Buffers:
         self._sizes = sizes
         self.storage = torch.empty(total, dtype=torch.uint8, device=device)
         base = self.storage.data_ptr()
-        self._struct = L.Book(*(base + o for o in self._off), self.rows, self.kv)
+        ptrs = [base + o for o in self._off]
+        self._struct = L.Book(*ptrs[:5], self.rows, self.kv, ptrs[5] if by_row else None)
         self._views = {}
 
     def struct(self) -> L.Book:
@@ -53,6 +57,8 @@ class _Buffers:
                 v = raw.view(torch.int16 if name == "tile_koff" else torch.int32)
                 if name == "tile_koff":
                     v = v.view(max(self.ntiles, 1), self.kv + 1)
+                if name == "tile_nbr":
+                    v = v.view(max(self.ntiles, 1), self.kv, L.TILE_ROWS) if self.by_row else None
                 self._views[name] = v
             return v
         raise AttributeError(name)
@@ -65,6 +71,11 @@ class _Buffers:
         own = self.grp_owner.view(self.ntiles, self.cap * L.GROUP)
         used = torch.arange(self.cap * L.GROUP, device=own.device)[None, :] < (ng * L.GROUP)[:, None]
         return int(((own >= 0) & used).sum().item())
+
+
+# Estimated pairs per stationary row from which a book also keeps its pairs by row (and the
+# convolution walks that form).  float("inf") never does, 0 always.
+BY_ROW_MIN_PAIRS = 6.0
 
 
 class RuleBook:
@@ -95,12 +106,22 @@ class RuleBook:
         return L.make_geom(self.batch, self.in_shape, self.out_shape, self.kernel, self.stride,
                            self.padding, self.dilation)
 
+    def _pairs_per_row(self, transposed: bool) -> float:
+        """Pairs a stationary row can expect: kernel volume x occupancy of the gathered side's grid
+        (a stride thins the offsets that can pair with an input row)."""
+        rows, shape = (self.out_rows, self.out_shape) if transposed else (self.in_rows, self.in_shape)
+        cells = max(self.batch * shape[0] * shape[1] * shape[2], 1)
+        est = self.kv * rows / cells
+        if transposed:
+            est /= self.stride[0] * self.stride[1] * self.stride[2]
+        return est
+
     def _build(self, transposed: bool, weight=None, weight_transposed: bool = False):
         """Launches the rule kernel.  With ``weight`` [KV,a,b] its fragment-ordered copy (what
         ``sph_weight_pack`` makes, for the contraction over ``a``, or over ``b`` when
         ``weight_transposed``) is produced by the same launch and returned with the buffers."""
         rows = self.in_rows if transposed else self.out_rows
-        buf = _Buffers(rows, self.kv, self.z_ptr.device)
+        buf = _Buffers(rows, self.kv, self.z_ptr.device, self._pairs_per_row(transposed) >= BY_ROW_MIN_PAIRS)
         g, b = self.geom(), buf.struct()
         lib = L.lib()
         if weight is None:

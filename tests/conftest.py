@@ -27,3 +27,15 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(params=["groups", "by_row"])
+def pair_form(request, monkeypatch):
+    """Runs a test once with the rule books in their grouped form only and once with the pairs also
+    kept by stationary row, which makes the convolution take its by-row kernel whatever the density."""
+    from sphconv_amd import rulebook
+    if request.param == "by_row":
+        monkeypatch.setattr(rulebook, "BY_ROW_MIN_PAIRS", 0.0)
+    else:
+        monkeypatch.setattr(rulebook, "BY_ROW_MIN_PAIRS", float("inf"))
+    return request.param

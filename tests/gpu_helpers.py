@@ -52,6 +52,22 @@ def book_triples(buf):
     return tri[order]
 
 
+def by_row_triples(buf):
+    """The by-row form of a book -> [P,3] (k, gather, owner) sorted by (k, owner); None if not kept."""
+    if buf.tile_nbr is None:
+        return None
+    torch.cuda.synchronize()
+    nt, kv = buf.ntiles, buf.kv
+    if nt == 0:
+        return np.zeros((0, 3), np.int64)
+    nbr = buf.tile_nbr[:nt].cpu().numpy()                      # [nt, kv, 128]
+    t, k, r = np.nonzero(nbr >= 0)
+    owner = t * L.TILE_ROWS + r
+    assert (owner < buf.rows).all()
+    tri = np.stack([k, nbr[t, k, r], owner], axis=1).astype(np.int64)
+    return tri[np.lexsort((tri[:, 2], tri[:, 0]))]
+
+
 def oracle_triples(rules, rule_size, swap=False):
     """Padded oracle rules -> [P,3] (k, in, out) sorted by (k, out)  (swap: (k, out, in) by (k, in))."""
     rules, rule_size = np.asarray(rules), np.asarray(rule_size)

@@ -16,7 +16,7 @@ import sphconv_amd
 from sphconv_amd import sphconv_cuda as ext
 from sphconv_amd.synth import make_config
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("pair_form")]
 CASES = H.load_ref_cases()
 
 

@@ -10,7 +10,7 @@ import sphconv_amd as sphconv
 from oracle import oracle as O
 from sphconv_amd.synth import make_config
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("pair_form")]
 
 
 def _inputs(seed, B, shape, C, p=0.2, dtype=torch.float32):

@@ -15,7 +15,7 @@ from sphconv_amd import sphconv_cuda as ext
 from sphconv_amd.rulebook import RuleBook
 from sphconv_amd.synth import make_config
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("pair_form")]
 CASES = H.load_ref_cases()
 
 
@@ -48,6 +48,10 @@ def _check(case, tile=(2, 2)):
     got_t = G.book_triples(book.transposed())
     assert np.array_equal(got_t, G.oracle_triples(rules, rule_size, swap=True))
     assert book.num_pairs() == want.shape[0]
+    # the same pairs by stationary row, where the book keeps that form
+    for buf, tri in ((book.fwd, want), (book.transposed(), got_t)):
+        rows = G.by_row_triples(buf)
+        assert rows is None or np.array_equal(rows, tri)
     # reference-format tensors
     p_rules, p_size = book.padded(tile)
     assert np.array_equal(p_size.cpu().numpy(), rule_size)
