@@ -509,94 +509,107 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
 // One wave per tile and 64 output columns; rows are requested half a tile (4 blocks)
 // ahead of their use.
 // ---------------------------------------------------------------------------
+constexpr int kRowsDepth = 4; // stages of gathered rows in flight per wave
+
 template <sph_dtype DT, int NS, int CT, bool MASKED>
-__global__ __launch_bounds__(128) void conv_rows_kernel(ConvArgs a, int nwtot)
+__device__ __forceinline__ void conv_rows_body(const ConvArgs &a, int nwtot)
 {
     typedef typename Traits<DT>::elem elem;
     typedef typename Traits<DT>::acc4 acc4;
-    constexpr int HB = R / SPH_GROUP / 2; // blocks of 16 rows per half tile
+    constexpr int NB = R / SPH_GROUP;     // blocks of 16 rows per tile
+    constexpr int BPS = NS >= 4 ? 1 : 4 / NS; // blocks per stage: a stage gathers BPS*NS = 4 sixteen-byte chunks per lane
+    constexpr int SPK = NB / BPS;         // stages per offset
+    constexpr int D = kRowsDepth;         // stages in flight
+    constexpr int U = (D > SPK) ? D : SPK; // stages per unrolled round (both are powers of two)
+    extern __shared__ __attribute__((aligned(16))) int32_t s_nb[]; // [KV][R] gathered row or -1
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
     const int tile = sph_xcd_tile(blockIdx.x, (a.book.rows + R - 1) / R);
     const int r0 = tile * R;
-    if (r0 >= a.book.rows) return;
+    if (r0 >= a.book.rows) return; // whole workgroups leave: no barrier is missed
     const int nrows = min(R, a.book.rows - r0);
     const int col0 = wave * CT * 16;
     const int KV = a.book.KV;
-    const int32_t *nb = a.book.tile_nbr + (long)tile * KV * R;
+    const int S = KV * SPK;
     const char *wlane = a.wp + ((long)(wave * CT)) * (kWave * 16) + lane * 16;
     const long wstep = (long)nwtot * (kWave * 16);
 
-    auto load_idx = [&](int k, int &lo, int &hi) { // rows 0..63 and 64..127 of offset k (clamped: always readable)
-        const int kk = min(k, KV - 1);
-        lo = nb[kk * R + lane];
-        hi = nb[kk * R + kWave + lane];
-    };
-    auto check_idx = [&](int &v) { v = (unsigned)v < (unsigned)a.feat_rows ? v : -1; };
-    auto issue_rows = [&](int sel, int4v (&fa)[HB][NS], int (&rows)[HB]) {
+    // the tile's table goes to LDS once (validated on the way): every stage then finds its rows
+    // with one LDS read per block instead of a dependent global load
+    {
+        const int4v *src = (const int4v *)(a.book.tile_nbr + (long)tile * KV * R);
+        for (int i = tid; i < KV * R / 4; i += blockDim.x) {
+            int4v v = src[i];
+            v.x = (unsigned)v.x < (unsigned)a.feat_rows ? v.x : -1;
+            v.y = (unsigned)v.y < (unsigned)a.feat_rows ? v.y : -1;
+            v.z = (unsigned)v.z < (unsigned)a.feat_rows ? v.z : -1;
+            v.w = (unsigned)v.w < (unsigned)a.feat_rows ? v.w : -1;
+            ((int4v *)s_nb)[i] = v;
+        }
+    }
+    __syncthreads();
+
+    int4v fa[D][BPS][NS], fw[NS][CT];
+    int rw[D][BPS];
+    acc4 acc[NB][CT];
 #pragma unroll
-        for (int j = 0; j < HB; j++) {
-            rows[j] = __shfl(sel, j * SPH_GROUP + (lane & 15), kWave);
+    for (int j = 0; j < NB; j++)
+#pragma unroll
+        for (int c = 0; c < CT; c++) acc[j][c] = acc4{0, 0, 0, 0};
+
+    // stage s = (k, q): offset k = s / SPK, blocks q*BPS .. q*BPS+BPS-1 of the tile, every 64-byte step of
+    // their rows (both halves of a 128-byte line are requested together); stages past the end re-read
+    // the last offset
+    auto issue = [&](int s, int q, int4v (&f)[BPS][NS], int (&rows)[BPS]) {
+        const int k = min(s / SPK, KV - 1);
+#pragma unroll
+        for (int j = 0; j < BPS; j++) {
+            rows[j] = s_nb[k * R + (q * BPS + j) * SPH_GROUP + (lane & 15)];
             const char *row = a.feat + (long)max(rows[j], 0) * a.row_bytes;
 #pragma unroll
             for (int st = 0; st < NS; st++) {
                 const int off = st * 64 + (lane >> 4) * 16;
-                fa[j][st] = *(const int4v *)(row + (off < a.row_bytes ? off : 0));
+                f[j][st] = *(const int4v *)(row + (off < a.row_bytes ? off : 0));
             }
         }
     };
-    auto load_w = [&](int k, int4v (&fw)[NS][CT]) {
-        const char *wk = wlane + (long)k * NS * wstep;
+    auto load_w = [&](int k) {
+        const char *wk = wlane + (long)min(k, KV - 1) * NS * wstep;
 #pragma unroll
         for (int st = 0; st < NS; st++)
 #pragma unroll
             for (int c = 0; c < CT; c++) fw[st][c] = *(const int4v *)(wk + st * wstep + (long)c * (kWave * 16));
     };
-    auto compute = [&](const int4v (&fw)[NS][CT], const int4v (&fa)[HB][NS], const int (&rows)[HB], acc4 (&ac)[HB][CT]) {
+
+    load_w(0);
 #pragma unroll
-        for (int j = 0; j < HB; j++)
+    for (int u = 0; u < D; u++) issue(u, u % SPK, fa[u], rw[u]);
+    for (int s0 = 0; s0 < S; s0 += U) {
 #pragma unroll
-            for (int st = 0; st < NS; st++) {
-                bool live = rows[j] >= 0;
-                if constexpr (MASKED) live = live && (st * 64 + (lane >> 4) * 16 < a.row_bytes);
-                const int4v x = live ? fa[j][st] : int4v{0, 0, 0, 0};
+        for (int u = 0; u < U; u++) {
+            const int s = s0 + u;
+            const int d = u % D, q = u % SPK; // compile-time after unrolling (U is a multiple of both)
+            __builtin_amdgcn_sched_barrier(0);
+            if (s < S) {
 #pragma unroll
-                for (int c = 0; c < CT; c++) ac[j][c] = mfma_step<DT>(fw[st][c], x, ac[j][c]);
+                for (int j = 0; j < BPS; j++)
+#pragma unroll
+                    for (int st = 0; st < NS; st++) {
+                        bool live = rw[d][j] >= 0;
+                        if constexpr (MASKED) live = live && (st * 64 + (lane >> 4) * 16 < a.row_bytes);
+                        const int4v x = live ? fa[d][j][st] : int4v{0, 0, 0, 0};
+#pragma unroll
+                        for (int c = 0; c < CT; c++) acc[q * BPS + j][c] = mfma_step<DT>(fw[st][c], x, acc[q * BPS + j][c]);
+                    }
             }
-    };
-
-    acc4 acc_lo[HB][CT], acc_hi[HB][CT];
-#pragma unroll
-    for (int j = 0; j < HB; j++)
-#pragma unroll
-        for (int c = 0; c < CT; c++) acc_lo[j][c] = acc_hi[j][c] = acc4{0, 0, 0, 0};
-
-    int lo, hi, lo_n, hi_n;
-    load_idx(0, lo, hi);
-    load_idx(1, lo_n, hi_n);
-    check_idx(lo);
-    check_idx(hi);
-    int4v fa0[HB][NS], fa1[HB][NS];
-    int rw0[HB], rw1[HB];
-    issue_rows(lo, fa0, rw0);
-    for (int k = 0; k < KV; k++) {
-        int4v fw[NS][CT];
-        load_w(k, fw);
-        issue_rows(hi, fa1, rw1);
-        __builtin_amdgcn_sched_barrier(0);
-        compute(fw, fa0, rw0, acc_lo);
-        __builtin_amdgcn_sched_barrier(0);
-        lo = lo_n;
-        hi = hi_n;
-        check_idx(lo);
-        check_idx(hi);
-        load_idx(k + 2, lo_n, hi_n);
-        issue_rows(lo, fa0, rw0); // first half of the next offset (of the last one again after the last: unused)
-        __builtin_amdgcn_sched_barrier(0);
-        compute(fw, fa1, rw1, acc_hi);
-        __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_sched_barrier(0);
+            // the offset is done: its weight registers take the next offset's fragments; the row buffers
+            // just consumed take stage s + D
+            if (q == SPK - 1) load_w(s / SPK + 1);
+            issue(s + D, (u + D) % SPK, fa[d], rw[d]);
+        }
     }
 
     // epilogue: a lane holds four consecutive columns of one row per block and column tile
@@ -635,9 +648,26 @@ __global__ __launch_bounds__(128) void conv_rows_kernel(ConvArgs a, int nwtot)
         }
     };
 #pragma unroll
-    for (int j = 0; j < HB; j++) store_block(j, acc_lo[j]);
-#pragma unroll
-    for (int j = 0; j < HB; j++) store_block(HB + j, acc_hi[j]);
+    for (int j = 0; j < NB; j++) store_block(j, acc[j]);
+}
+
+// The accumulators of a wave are CT*32 registers; the wrappers tell the compiler how many waves per
+// SIMD to leave room for (4 column tiles: 2, 2 tiles: 3, 1 tile: 4), i.e. how many registers the
+// gathers in flight may take.
+template <sph_dtype DT, int NS, int CT, bool MASKED>
+__global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2))) void conv_rows_kernel_w2(ConvArgs a, int nwtot)
+{
+    conv_rows_body<DT, NS, CT, MASKED>(a, nwtot);
+}
+template <sph_dtype DT, int NS, int CT, bool MASKED>
+__global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(3))) void conv_rows_kernel_w3(ConvArgs a, int nwtot)
+{
+    conv_rows_body<DT, NS, CT, MASKED>(a, nwtot);
+}
+template <sph_dtype DT, int NS, int CT, bool MASKED>
+__global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(4))) void conv_rows_kernel_w4(ConvArgs a, int nwtot)
+{
+    conv_rows_body<DT, NS, CT, MASKED>(a, nwtot);
 }
 
 // ---------------------------------------------------------------------------
@@ -1125,15 +1155,23 @@ int launch_conv_wave_ct(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st
     }
 }
 
+template <sph_dtype DT, int NS, int CT, bool MASKED>
+int launch_conv_rows_m(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
+{
+    const int waves = (nwtot + CT - 1) / CT;
+    const size_t lds = (size_t)a.book.KV * R * sizeof(int32_t);
+    const dim3 grid(sph_xcd_grid(ntiles)), block(waves * kWave);
+    if constexpr (CT >= 4) hipLaunchKernelGGL((conv_rows_kernel_w2<DT, NS, CT, MASKED>), grid, block, lds, st, a, nwtot);
+    else if constexpr (CT == 2) hipLaunchKernelGGL((conv_rows_kernel_w3<DT, NS, CT, MASKED>), grid, block, lds, st, a, nwtot);
+    else hipLaunchKernelGGL((conv_rows_kernel_w4<DT, NS, CT, MASKED>), grid, block, lds, st, a, nwtot);
+    return sph_check_launch("sph_conv_apply");
+}
+
 template <sph_dtype DT, int NS, int CT>
 int launch_conv_rows(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
 {
-    const int waves = (nwtot + CT - 1) / CT;
-    if (a.row_bytes < NS * 64)
-        hipLaunchKernelGGL((conv_rows_kernel<DT, NS, CT, true>), dim3(sph_xcd_grid(ntiles)), dim3(waves * kWave), 0, st, a, nwtot);
-    else
-        hipLaunchKernelGGL((conv_rows_kernel<DT, NS, CT, false>), dim3(sph_xcd_grid(ntiles)), dim3(waves * kWave), 0, st, a, nwtot);
-    return sph_check_launch("sph_conv_apply");
+    if (a.row_bytes < NS * 64) return launch_conv_rows_m<DT, NS, CT, true>(a, nwtot, ntiles, st);
+    return launch_conv_rows_m<DT, NS, CT, false>(a, nwtot, ntiles, st);
 }
 
 template <sph_dtype DT, int NS>
@@ -1149,11 +1187,12 @@ int launch_conv_rows_ct(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st
 template <sph_dtype DT, int NW>
 int launch_conv(const ConvArgs &a, int ntiles, hipStream_t st)
 {
-    if (a.aligned_in && a.aligned_out && a.feat_rows > 0 && a.book.tile_nbr) {
-        switch (a.nsteps) {
+    // by stationary row, when the book keeps that form (its table must fit the default 64 KiB of LDS)
+    if (a.aligned_in && a.aligned_out && a.feat_rows > 0 && a.book.tile_nbr &&
+        (size_t)a.book.KV * R * sizeof(int32_t) <= 64 * 1024 && (uintptr_t)a.book.tile_nbr % 16 == 0) {
+        switch (a.nsteps) { // rows of up to 128 bytes; longer ones (4 steps of weight fragments) go by groups
         case 1: return launch_conv_rows_ct<DT, 1>(a, NW, ntiles, st);
         case 2: return launch_conv_rows_ct<DT, 2>(a, NW, ntiles, st);
-        case 4: return launch_conv_rows_ct<DT, 4>(a, NW, ntiles, st);
         default: break;
         }
     }

@@ -75,7 +75,7 @@ class _Buffers:
 
 # Estimated pairs per stationary row from which a book also keeps its pairs by row (and the
 # convolution walks that form).  float("inf") never does, 0 always.
-BY_ROW_MIN_PAIRS = 6.0
+BY_ROW_MIN_PAIRS = 10.0
 
 
 class RuleBook:
