@@ -509,8 +509,6 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
 // One wave per tile and 64 output columns; rows are requested half a tile (4 blocks)
 // ahead of their use.
 // ---------------------------------------------------------------------------
-constexpr int kRowsDepth = 4; // stages of gathered rows in flight per wave
-
 template <sph_dtype DT, int NS, int CT, bool MASKED>
 __device__ __forceinline__ void conv_rows_body(const ConvArgs &a, int nwtot)
 {
@@ -519,8 +517,11 @@ __device__ __forceinline__ void conv_rows_body(const ConvArgs &a, int nwtot)
     constexpr int NB = R / SPH_GROUP;     // blocks of 16 rows per tile
     constexpr int BPS = NS >= 4 ? 1 : 4 / NS; // blocks per stage: a stage gathers BPS*NS = 4 sixteen-byte chunks per lane
     constexpr int SPK = NB / BPS;         // stages per offset
-    constexpr int D = kRowsDepth;         // stages in flight
-    constexpr int U = (D > SPK) ? D : SPK; // stages per unrolled round (both are powers of two)
+    // measured: 128-byte rows want four stages of gathers in flight and one set of weight registers; 64-byte
+    // rows (few MFMAs per stage) two stages and the next offset's weights requested an offset ahead
+    constexpr int D = NS >= 2 ? 4 : 2;    // stages in flight
+    constexpr int KW = NS >= 2 ? 1 : 2;   // sets of weight fragment registers
+    constexpr int U = (D > SPK * KW) ? D : SPK * KW; // stages per unrolled round (all powers of two)
     extern __shared__ __attribute__((aligned(16))) int32_t s_nb[]; // [KV][R] gathered row or -1
 
     const int tid = threadIdx.x;
@@ -551,8 +552,17 @@ __device__ __forceinline__ void conv_rows_body(const ConvArgs &a, int nwtot)
     }
     __syncthreads();
 
-    int4v fa[D][BPS][NS], fw[NS][CT];
-    int rw[D][BPS];
+    // Gathers are requested with the four lanes of a quad on the four 16-byte chunks of ONE row's 64-byte
+    // step (one tag look-up per quad; with a lane per row of the MFMA layout every quad would touch four
+    // rows).  They reach the MFMA layout (lane = pair + 16 * chunk) through a wave-private LDS buffer:
+    // [chunk set][16 rows][80 bytes] (the 16-byte pad makes both the write and the read conflict-free).
+    // With 64-byte rows (one step) the exchange costs more than the look-ups it saves: there a lane loads
+    // its MFMA operand directly.
+    constexpr bool QUAD = NS >= 2;
+    constexpr int kTrRow = 80, kTrSet = SPH_GROUP * kTrRow;
+    char *tr = (char *)(s_nb + KV * R) + wave * (BPS * NS * kTrSet);
+    int4v fa[D][BPS][NS], fw[KW][NS][CT];
+    int rq[D][BPS];
     acc4 acc[NB][CT];
 #pragma unroll
     for (int j = 0; j < NB; j++)
@@ -560,55 +570,73 @@ __device__ __forceinline__ void conv_rows_body(const ConvArgs &a, int nwtot)
         for (int c = 0; c < CT; c++) acc[j][c] = acc4{0, 0, 0, 0};
 
     // stage s = (k, q): offset k = s / SPK, blocks q*BPS .. q*BPS+BPS-1 of the tile, every 64-byte step of
-    // their rows (both halves of a 128-byte line are requested together); stages past the end re-read
-    // the last offset
+    // their rows; stages past the end re-read the last offset
     auto issue = [&](int s, int q, int4v (&f)[BPS][NS], int (&rows)[BPS]) {
         const int k = min(s / SPK, KV - 1);
 #pragma unroll
         for (int j = 0; j < BPS; j++) {
-            rows[j] = s_nb[k * R + (q * BPS + j) * SPH_GROUP + (lane & 15)];
+            rows[j] = s_nb[k * R + (q * BPS + j) * SPH_GROUP + (QUAD ? lane >> 2 : lane & 15)];
             const char *row = a.feat + (long)max(rows[j], 0) * a.row_bytes;
 #pragma unroll
             for (int st = 0; st < NS; st++) {
-                const int off = st * 64 + (lane >> 4) * 16;
+                const int off = st * 64 + (QUAD ? lane & 3 : lane >> 4) * 16;
                 f[j][st] = *(const int4v *)(row + (off < a.row_bytes ? off : 0));
             }
         }
     };
-    auto load_w = [&](int k) {
+    auto load_w = [&](int k, int4v (&w)[NS][CT]) {
         const char *wk = wlane + (long)min(k, KV - 1) * NS * wstep;
 #pragma unroll
         for (int st = 0; st < NS; st++)
 #pragma unroll
-            for (int c = 0; c < CT; c++) fw[st][c] = *(const int4v *)(wk + st * wstep + (long)c * (kWave * 16));
+            for (int c = 0; c < CT; c++) w[st][c] = *(const int4v *)(wk + st * wstep + (long)c * (kWave * 16));
     };
 
-    load_w(0);
 #pragma unroll
-    for (int u = 0; u < D; u++) issue(u, u % SPK, fa[u], rw[u]);
+    for (int p = 0; p < KW; p++) load_w(p, fw[p]);
+#pragma unroll
+    for (int u = 0; u < D; u++) issue(u, u % SPK, fa[u], rq[u]);
     for (int s0 = 0; s0 < S; s0 += U) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int s = s0 + u;
-            const int d = u % D, q = u % SPK; // compile-time after unrolling (U is a multiple of both)
+            const int d = u % D, q = u % SPK, p = (u / SPK) % KW; // compile-time after unrolling
             __builtin_amdgcn_sched_barrier(0);
             if (s < S) {
+                // zeros for rows without a pair and beyond the row's end; quad layout -> LDS -> MFMA layout
+                int4v x[BPS][NS];
 #pragma unroll
                 for (int j = 0; j < BPS; j++)
 #pragma unroll
                     for (int st = 0; st < NS; st++) {
-                        bool live = rw[d][j] >= 0;
-                        if constexpr (MASKED) live = live && (st * 64 + (lane >> 4) * 16 < a.row_bytes);
-                        const int4v x = live ? fa[d][j][st] : int4v{0, 0, 0, 0};
-#pragma unroll
-                        for (int c = 0; c < CT; c++) acc[q * BPS + j][c] = mfma_step<DT>(fw[st][c], x, acc[q * BPS + j][c]);
+                        bool live = rq[d][j] >= 0;
+                        if constexpr (MASKED) live = live && (st * 64 + (QUAD ? lane & 3 : lane >> 4) * 16 < a.row_bytes);
+                        x[j][st] = live ? fa[d][j][st] : int4v{0, 0, 0, 0};
+                        if constexpr (QUAD)
+                            *(int4v *)(tr + (j * NS + st) * kTrSet + (lane >> 2) * kTrRow + (lane & 3) * 16) = x[j][st];
                     }
+                if constexpr (QUAD) {
+                    asm volatile("" ::: "memory"); // other lanes' chunks: keep the reads behind the writes
+#pragma unroll
+                    for (int j = 0; j < BPS; j++)
+#pragma unroll
+                        for (int st = 0; st < NS; st++)
+                            x[j][st] = *(const int4v *)(tr + (j * NS + st) * kTrSet + (lane & 15) * kTrRow + (lane >> 4) * 16);
+                }
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int j = 0; j < BPS; j++)
+#pragma unroll
+                    for (int st = 0; st < NS; st++)
+#pragma unroll
+                        for (int c = 0; c < CT; c++)
+                            acc[q * BPS + j][c] = mfma_step<DT>(fw[p][st][c], x[j][st], acc[q * BPS + j][c]);
             }
             __builtin_amdgcn_sched_barrier(0);
-            // the offset is done: its weight registers take the next offset's fragments; the row buffers
+            // the offset is done: its weight registers take the fragments of offset k + KW; the row buffers
             // just consumed take stage s + D
-            if (q == SPK - 1) load_w(s / SPK + 1);
-            issue(s + D, (u + D) % SPK, fa[d], rw[d]);
+            if (q == SPK - 1) load_w(s / SPK + KW, fw[p]);
+            issue(s + D, (u + D) % SPK, fa[d], rq[d]);
         }
     }
 
@@ -1159,7 +1187,8 @@ template <sph_dtype DT, int NS, int CT, bool MASKED>
 int launch_conv_rows_m(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
 {
     const int waves = (nwtot + CT - 1) / CT;
-    const size_t lds = (size_t)a.book.KV * R * sizeof(int32_t);
+    // the table, and for 128-byte rows a wave's exchange buffer (4 chunk sets of 16 rows x 80 bytes)
+    const size_t lds = (size_t)a.book.KV * R * sizeof(int32_t) + (NS >= 2 ? (size_t)waves * 4 * SPH_GROUP * 80 : 0);
     const dim3 grid(sph_xcd_grid(ntiles)), block(waves * kWave);
     if constexpr (CT >= 4) hipLaunchKernelGGL((conv_rows_kernel_w2<DT, NS, CT, MASKED>), grid, block, lds, st, a, nwtot);
     else if constexpr (CT == 2) hipLaunchKernelGGL((conv_rows_kernel_w3<DT, NS, CT, MASKED>), grid, block, lds, st, a, nwtot);
@@ -1189,7 +1218,7 @@ int launch_conv(const ConvArgs &a, int ntiles, hipStream_t st)
 {
     // by stationary row, when the book keeps that form (its table must fit the default 64 KiB of LDS)
     if (a.aligned_in && a.aligned_out && a.feat_rows > 0 && a.book.tile_nbr &&
-        (size_t)a.book.KV * R * sizeof(int32_t) <= 64 * 1024 && (uintptr_t)a.book.tile_nbr % 16 == 0) {
+        (size_t)a.book.KV * R * sizeof(int32_t) <= 48 * 1024 && (uintptr_t)a.book.tile_nbr % 16 == 0) {
         switch (a.nsteps) { // rows of up to 128 bytes; longer ones (4 steps of weight fragments) go by groups
         case 1: return launch_conv_rows_ct<DT, 1>(a, NW, ntiles, st);
         case 2: return launch_conv_rows_ct<DT, 2>(a, NW, ntiles, st);
