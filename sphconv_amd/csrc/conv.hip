@@ -513,24 +513,31 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
 // Measured at 64->64 fp16 on a full grid: 164 us against 387 us by groups; without any
 // load the same instruction stream takes 91 us (one MFMA issues per 32 cycles and SIMD).
 // ---------------------------------------------------------------------------
-template <sph_dtype DT, int NS, int CT, bool MASKED>
+// WS = waves that share a tile's rows (1, or 4 when the grid has fewer tiles than the chip has SIMDs: the
+// kernel then lasts as long as one wave's chain of KV * 8 steps, and four waves with two blocks each
+// shorten it).
+template <sph_dtype DT, int NS, int CT, bool MASKED, int WS>
 __device__ __forceinline__ void conv_rows_body(const ConvArgs &a, int nwtot)
 {
     typedef typename Traits<DT>::elem elem;
     typedef typename Traits<DT>::acc4 acc4;
-    constexpr int NB = R / SPH_GROUP;     // blocks of 16 rows per tile
-    constexpr int BPS = NS >= 4 ? 1 : 4 / NS; // blocks per stage: a stage gathers BPS*NS = 4 sixteen-byte chunks per lane
+    constexpr int NB = R / SPH_GROUP / WS; // blocks of 16 rows per wave
+    constexpr int BPS0 = NS >= 4 ? 1 : 4 / NS;
+    constexpr int BPS = BPS0 < NB ? BPS0 : NB; // blocks per stage: a stage gathers up to 4 sixteen-byte chunks per lane
     constexpr int SPK = NB / BPS;         // stages per offset
     // measured: 128-byte rows want four stages of gathers in flight and one set of weight registers; 64-byte
-    // rows (few MFMAs per stage) two stages and the next offset's weights requested an offset ahead
-    constexpr int D = NS >= 2 ? 4 : 2;    // stages in flight
-    constexpr int KW = NS >= 2 ? 1 : 2;   // sets of weight fragment registers
+    // rows (few MFMAs per stage) two stages and the next offset's weights requested an offset ahead; a
+    // wave that takes a quarter of the rows has the registers for four offsets of weights
+    constexpr int D = (NS >= 2 || WS > 1) ? 4 : 2; // stages in flight
+    constexpr int KW = WS > 1 ? 4 / SPK : (NS >= 2 ? 1 : 2); // sets of weight fragment registers
     constexpr int U = (D > SPK * KW) ? D : SPK * KW; // stages per unrolled round (all powers of two)
     extern __shared__ __attribute__((aligned(16))) int32_t s_nb[]; // [KV][R] gathered row or -1
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
-    const int wave = tid / kWave;
+    const int wave = tid / kWave / WS;         // block of CT*16 columns
+    const int part = (tid / kWave) % WS;       // which blocks of the tile
+    const int blk0 = part * NB;
     const int tile = sph_xcd_tile(blockIdx.x, (a.book.rows + R - 1) / R);
     const int r0 = tile * R;
     if (r0 >= a.book.rows) return; // whole workgroups leave: no barrier is missed
@@ -564,7 +571,7 @@ __device__ __forceinline__ void conv_rows_body(const ConvArgs &a, int nwtot)
     // its MFMA operand directly.
     constexpr bool QUAD = NS >= 2;
     constexpr int kTrRow = 80, kTrSet = SPH_GROUP * kTrRow;
-    char *tr = (char *)(s_nb + KV * R) + wave * (BPS * NS * kTrSet);
+    char *tr = (char *)(s_nb + KV * R) + (tid / kWave) * (BPS * NS * kTrSet);
     int4v fa[D][BPS][NS], fw[KW][NS][CT];
     int rq[D][BPS];
     acc4 acc[NB][CT];
@@ -579,7 +586,7 @@ __device__ __forceinline__ void conv_rows_body(const ConvArgs &a, int nwtot)
         const int k = min(s / SPK, KV - 1);
 #pragma unroll
         for (int j = 0; j < BPS; j++) {
-            rows[j] = s_nb[k * R + (q * BPS + j) * SPH_GROUP + (QUAD ? lane >> 2 : lane & 15)];
+            rows[j] = s_nb[k * R + (blk0 + q * BPS + j) * SPH_GROUP + (QUAD ? lane >> 2 : lane & 15)];
             const char *row = a.feat + (long)max(rows[j], 0) * a.row_bytes;
 #pragma unroll
             for (int st = 0; st < NS; st++) {
@@ -680,7 +687,7 @@ __device__ __forceinline__ void conv_rows_body(const ConvArgs &a, int nwtot)
         }
     };
 #pragma unroll
-    for (int j = 0; j < NB; j++) store_block(j, acc[j]);
+    for (int j = 0; j < NB; j++) store_block(blk0 + j, acc[j]);
 }
 
 // The accumulators of a wave are CT*32 registers; the wrappers tell the compiler how many waves per
@@ -689,17 +696,23 @@ __device__ __forceinline__ void conv_rows_body(const ConvArgs &a, int nwtot)
 template <sph_dtype DT, int NS, int CT, bool MASKED>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2))) void conv_rows_kernel_w2(ConvArgs a, int nwtot)
 {
-    conv_rows_body<DT, NS, CT, MASKED>(a, nwtot);
+    conv_rows_body<DT, NS, CT, MASKED, 1>(a, nwtot);
 }
 template <sph_dtype DT, int NS, int CT, bool MASKED>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(3))) void conv_rows_kernel_w3(ConvArgs a, int nwtot)
 {
-    conv_rows_body<DT, NS, CT, MASKED>(a, nwtot);
+    conv_rows_body<DT, NS, CT, MASKED, 1>(a, nwtot);
 }
 template <sph_dtype DT, int NS, int CT, bool MASKED>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(4))) void conv_rows_kernel_w4(ConvArgs a, int nwtot)
 {
-    conv_rows_body<DT, NS, CT, MASKED>(a, nwtot);
+    conv_rows_body<DT, NS, CT, MASKED, 1>(a, nwtot);
+}
+// four waves per tile and block of columns
+template <sph_dtype DT, int NS, int CT, bool MASKED>
+__global__ __launch_bounds__(512) void conv_rows_kernel_split(ConvArgs a, int nwtot)
+{
+    conv_rows_body<DT, NS, CT, MASKED, 4>(a, nwtot);
 }
 
 // ---------------------------------------------------------------------------
@@ -1191,10 +1204,13 @@ template <sph_dtype DT, int NS, int CT, bool MASKED>
 int launch_conv_rows_m(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
 {
     const int waves = (nwtot + CT - 1) / CT;
-    // the table, and for 128-byte rows a wave's exchange buffer (4 chunk sets of 16 rows x 80 bytes)
-    const size_t lds = (size_t)a.book.KV * R * sizeof(int32_t) + (NS >= 2 ? (size_t)waves * 4 * SPH_GROUP * 80 : 0);
-    const dim3 grid(sph_xcd_grid(ntiles)), block(waves * kWave);
-    if constexpr (CT >= 4) hipLaunchKernelGGL((conv_rows_kernel_w2<DT, NS, CT, MASKED>), grid, block, lds, st, a, nwtot);
+    // fewer tiles than SIMDs: the kernel lasts one wave's chain, so four waves share a tile's rows
+    const int ws = ntiles <= 1024 ? 4 : 1;
+    // the table, and for 128-byte rows a wave's exchange buffer (up to 4 chunk sets of 16 rows x 80 bytes)
+    const size_t lds = (size_t)a.book.KV * R * sizeof(int32_t) + (NS >= 2 ? (size_t)waves * ws * 4 * SPH_GROUP * 80 : 0);
+    const dim3 grid(sph_xcd_grid(ntiles)), block(waves * ws * kWave);
+    if (ws == 4) hipLaunchKernelGGL((conv_rows_kernel_split<DT, NS, CT, MASKED>), grid, block, lds, st, a, nwtot);
+    else if constexpr (CT >= 4) hipLaunchKernelGGL((conv_rows_kernel_w2<DT, NS, CT, MASKED>), grid, block, lds, st, a, nwtot);
     else if constexpr (CT == 2) hipLaunchKernelGGL((conv_rows_kernel_w3<DT, NS, CT, MASKED>), grid, block, lds, st, a, nwtot);
     else hipLaunchKernelGGL((conv_rows_kernel_w4<DT, NS, CT, MASKED>), grid, block, lds, st, a, nwtot);
     return sph_check_launch("sph_conv_apply");
