@@ -89,7 +89,11 @@ typedef struct sph_book {
      * gathered row of (tile, offset, row of the tile) or -1.  When not null, sph_rules_build*
      * and sph_rules_from_padded fill it too, and sph_conv_apply walks it instead of the groups
      * (every offset of every block of 16 rows costs one step, whatever it holds: the faster
-     * way from about six pairs per row upwards).  Null: not kept. */
+     * way from about ten pairs per row upwards).  Null: not kept.
+     * A book that keeps this table may leave grp_k, grp_gather and grp_owner null (all three):
+     * the rule kernel then writes only the counts and the table, sph_conv_apply serves the calls
+     * it can walk by rows (rows of 16-byte multiples up to 128 bytes) and refuses the others,
+     * sph_conv_wgrad and sph_rules_to_padded_count refuse the book. */
     int32_t *tile_nbr;
 } sph_book;
 

@@ -105,6 +105,13 @@ struct ConvArgs {
     int aligned_in, aligned_out;
 };
 
+// can sph_conv_apply walk this call by stationary row?
+inline bool rows_path_ok(const ConvArgs &a)
+{
+    return a.aligned_in && a.aligned_out && a.feat_rows > 0 && a.book.tile_nbr && (a.nsteps == 1 || a.nsteps == 2) &&
+           (size_t)a.book.KV * R * sizeof(int32_t) <= 48 * 1024 && (uintptr_t)a.book.tile_nbr % 16 == 0;
+}
+
 template <sph_dtype DT>
 __device__ __forceinline__ int4v load_a_frag(const ConvArgs &a, int in_row, int st, int lane)
 {
@@ -1236,14 +1243,10 @@ int launch_conv_rows_ct(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st
 template <sph_dtype DT, int NW>
 int launch_conv(const ConvArgs &a, int ntiles, hipStream_t st)
 {
-    // by stationary row, when the book keeps that form (its table must fit the default 64 KiB of LDS)
-    if (a.aligned_in && a.aligned_out && a.feat_rows > 0 && a.book.tile_nbr &&
-        (size_t)a.book.KV * R * sizeof(int32_t) <= 48 * 1024 && (uintptr_t)a.book.tile_nbr % 16 == 0) {
-        switch (a.nsteps) { // rows of up to 128 bytes; longer ones (4 steps of weight fragments) go by groups
-        case 1: return launch_conv_rows_ct<DT, 1>(a, NW, ntiles, st);
-        case 2: return launch_conv_rows_ct<DT, 2>(a, NW, ntiles, st);
-        default: break;
-        }
+    // by stationary row, when the book keeps that form (rows of up to 128 bytes; its table must fit LDS)
+    if (rows_path_ok(a)) {
+        if (a.nsteps == 1) return launch_conv_rows_ct<DT, 1>(a, NW, ntiles, st);
+        return launch_conv_rows_ct<DT, 2>(a, NW, ntiles, st);
     }
     if (a.aligned_in && a.feat_rows > 0) {
         switch (a.nsteps) {
@@ -1336,10 +1339,13 @@ int launch_wgrad(const WgradArgs &a0, void *dw, hipStream_t st)
     return sph_check_launch("sph_conv_wgrad(reduce)");
 }
 
+inline int book_has_groups(const sph_book *b) { return b->grp_k && b->grp_gather && b->grp_owner; }
+
+// the groups may be missing (all three arrays null) in a book that keeps its pairs by row
 inline int book_ok(const sph_book *b)
 {
-    return b && b->tile_ngrp && b->tile_koff && b->grp_k && b->grp_gather && b->grp_owner &&
-           b->rows >= 0 && b->KV > 0 && b->KV <= SPH_MAX_KV;
+    return b && b->tile_ngrp && b->tile_koff && b->rows >= 0 && b->KV > 0 && b->KV <= SPH_MAX_KV &&
+           (book_has_groups(b) || (b->tile_nbr && !b->grp_k && !b->grp_gather && !b->grp_owner));
 }
 
 } // namespace
@@ -1391,6 +1397,9 @@ SPH_EXPORT int sph_conv_apply(sph_dtype dt, const void *feature, int feature_row
     a.aligned_in = (a.row_bytes % 16 == 0) && ((uintptr_t)feature % 16 == 0);
     a.aligned_out = ((ndim * es) % 16 == 0) && ((uintptr_t)out % 16 == 0);
     SPH_REQUIRE((uintptr_t)packed_w % 16 == 0, SPH_ERR_ARG, "sph_conv_apply: packed weight must be 16-byte aligned");
+    SPH_REQUIRE(book_has_groups(book) || rows_path_ok(a), SPH_ERR_ARG,
+                "sph_conv_apply: the book holds no groups and this call cannot go by rows (rows of 16-byte multiples up to "
+                "128 bytes, 16-byte aligned arrays)");
     const int nw = pad_waves(ndim), nt = sph_book_tiles(book->rows);
     hipStream_t st = (hipStream_t)stream;
     switch (dt) {
@@ -1415,7 +1424,7 @@ SPH_EXPORT size_t sph_wgrad_partial_elems(int KV, int iC, int oC, int out_rows)
 SPH_EXPORT int sph_conv_wgrad(sph_dtype dt, const void *feature, int in_rows, int iC, const void *d_out,
                               int oC, const sph_book *fwd_book, float *partial, void *d_weight, void *stream)
 {
-    SPH_REQUIRE(book_ok(fwd_book), SPH_ERR_ARG, "sph_conv_wgrad: bad book");
+    SPH_REQUIRE(book_ok(fwd_book) && book_has_groups(fwd_book), SPH_ERR_ARG, "sph_conv_wgrad: bad book (it must hold its groups)");
     SPH_REQUIRE(partial && d_weight, SPH_ERR_ARG, "sph_conv_wgrad: null pointer");
     SPH_REQUIRE(dt == SPH_F32 || dt == SPH_F16 || dt == SPH_BF16, SPH_ERR_UNSUPPORTED,
                 "sph_conv_wgrad: dtype %d has no weight gradient", (int)dt);

@@ -167,6 +167,9 @@ __device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int t
     }
     __syncthreads();
 
+    for (int k = tid; k <= KV; k += kThreads)
+        book.tile_koff[(long)tile * (KV + 1) + k] = (uint16_t)sc.goff[k];
+    if (!book.grp_gather) return; // the caller keeps the pairs by row only: counts are written, groups are not
     const int ngrp = sc.goff[KV];
     const long gbase_tile = (long)tile * cap;
     for (int slot = tid; slot < ngrp * SPH_GROUP; slot += kThreads) {
@@ -185,8 +188,6 @@ __device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int t
         book.grp_owner[gbase_tile * SPH_GROUP + slot] = own;
     }
     for (int g = tid; g < ngrp; g += kThreads) book.grp_k[gbase_tile + g] = sc.gk[g];
-    for (int k = tid; k <= KV; k += kThreads)
-        book.tile_koff[(long)tile * (KV + 1) + k] = (uint16_t)sc.goff[k];
 }
 
 // ---------------------------------------------------------------------------
@@ -670,10 +671,13 @@ inline ConvParams conv_params(const sph_geom *g)
                       g->pad[0], g->pad[1], g->pad[2]};
 }
 
+inline int book_has_groups(const sph_book *b) { return b->grp_k && b->grp_gather && b->grp_owner; }
+
+// the groups may be left out (all three arrays null) by a caller that keeps the pairs by row
 inline int book_ok(const sph_book *b)
 {
-    return b && b->tile_ngrp && b->tile_koff && b->grp_k && b->grp_gather && b->grp_owner &&
-           b->rows >= 0 && b->KV > 0 && b->KV <= SPH_MAX_KV;
+    return b && b->tile_ngrp && b->tile_koff && b->rows >= 0 && b->KV > 0 && b->KV <= SPH_MAX_KV &&
+           (book_has_groups(b) || (b->tile_nbr && !b->grp_k && !b->grp_gather && !b->grp_owner));
 }
 
 } // namespace
@@ -872,7 +876,8 @@ SPH_EXPORT int sph_rules_to_padded_count(const sph_book *fwd_book, const int32_t
                                          int32_t *rule_size, void *stream)
 {
     SPH_REQUIRE(sph_geom_ok(g) && T0 > 0 && T1 > 0, SPH_ERR_ARG, "sph_rules_to_padded_count: bad geometry");
-    SPH_REQUIRE(book_ok(fwd_book) && oz_ptr && nbr && rule_size, SPH_ERR_ARG, "sph_rules_to_padded_count: null argument");
+    SPH_REQUIRE(book_ok(fwd_book) && book_has_groups(fwd_book) && oz_ptr && nbr && rule_size, SPH_ERR_ARG,
+                "sph_rules_to_padded_count: null argument (the book must hold its groups)");
     hipStream_t st = (hipStream_t)stream;
     const int KV = fwd_book->KV, rows = fwd_book->rows;
     const int nt = sph_book_tiles(rows), cap = sph_book_cap(KV);

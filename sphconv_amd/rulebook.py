@@ -21,17 +21,20 @@ class _Buffers:
 
     _FIELDS = ("tile_ngrp", "tile_koff", "grp_k", "grp_gather", "grp_owner", "tile_nbr")
 
-    def __init__(self, rows: int, kv: int, device, by_row: bool = False):
+    def __init__(self, rows: int, kv: int, device, by_row: bool = False, groups: bool = True):
         """``by_row`` also keeps the pairs by stationary row (``tile_nbr`` [NT,KV,128]), the form the
-        convolution walks when neighbourhoods are dense."""
+        convolution walks when neighbourhoods are dense; with it, ``groups=False`` leaves the groups out
+        (forward-only use: the rule kernel then writes a fifth of the bytes)."""
         lib = L.lib()
         self.rows, self.kv = int(rows), int(kv)
         self.ntiles = lib.sph_book_tiles(self.rows)
         self.cap = lib.sph_book_cap(self.kv)
         self.by_row = bool(by_row)
+        self.groups = bool(groups) or not self.by_row
         nt = max(self.ntiles, 1)
-        sizes = (nt * 4, nt * (self.kv + 1) * 2, nt * self.cap * 4, nt * self.cap * L.GROUP * 4,
-                 nt * self.cap * L.GROUP * 4, nt * self.kv * L.TILE_ROWS * 4 if by_row else 0)
+        g = 1 if self.groups else 0
+        sizes = (nt * 4, nt * (self.kv + 1) * 2, g * nt * self.cap * 4, g * nt * self.cap * L.GROUP * 4,
+                 g * nt * self.cap * L.GROUP * 4, nt * self.kv * L.TILE_ROWS * 4 if by_row else 0)
         self._off = []
         total = 0
         for sz in sizes:
@@ -41,6 +44,8 @@ class _Buffers:
         self.storage = torch.empty(total, dtype=torch.uint8, device=device)
         base = self.storage.data_ptr()
         ptrs = [base + o for o in self._off]
+        if not self.groups:
+            ptrs[2] = ptrs[3] = ptrs[4] = None
         self._struct = L.Book(*ptrs[:5], self.rows, self.kv, ptrs[5] if by_row else None)
         self._views = {}
 
@@ -59,6 +64,8 @@ class _Buffers:
                     v = v.view(max(self.ntiles, 1), self.kv + 1)
                 if name == "tile_nbr":
                     v = v.view(max(self.ntiles, 1), self.kv, L.TILE_ROWS) if self.by_row else None
+                elif name.startswith("grp_") and not self.groups:
+                    v = None
                 self._views[name] = v
             return v
         raise AttributeError(name)
@@ -67,6 +74,8 @@ class _Buffers:
         """Total pairs held (synchronises)."""
         if self.ntiles == 0:
             return 0
+        if not self.groups:
+            return int((self.tile_nbr[:self.ntiles] >= 0).sum().item())
         ng = self.tile_ngrp[:self.ntiles].long()
         own = self.grp_owner.view(self.ntiles, self.cap * L.GROUP)
         used = torch.arange(self.cap * L.GROUP, device=own.device)[None, :] < (ng * L.GROUP)[:, None]
@@ -116,12 +125,27 @@ class RuleBook:
             est /= self.stride[0] * self.stride[1] * self.stride[2]
         return est
 
-    def _build(self, transposed: bool, weight=None, weight_transposed: bool = False):
+    def _rows_kernel_takes(self, weight, weight_transposed: bool) -> bool:
+        """Whether ``sph_conv_apply`` can walk this layer by stationary row (rows of 16-byte multiples up
+        to 128 bytes, 16-byte multiples out, a table that fits LDS): the conditions of the library."""
+        kv, wa, wb = weight.shape
+        kdim, ndim = (wb, wa) if weight_transposed else (wa, wb)
+        es = weight.element_size()
+        return (kdim * es) % 16 == 0 and kdim * es <= 128 and (ndim * es) % 16 == 0 and kv * L.TILE_ROWS * 4 <= 48 * 1024
+
+    def _build(self, transposed: bool, weight=None, weight_transposed: bool = False, groups: Optional[bool] = None):
         """Launches the rule kernel.  With ``weight`` [KV,a,b] its fragment-ordered copy (what
         ``sph_weight_pack`` makes, for the contraction over ``a``, or over ``b`` when
-        ``weight_transposed``) is produced by the same launch and returned with the buffers."""
+        ``weight_transposed``) is produced by the same launch and returned with the buffers.
+        ``groups`` None: a by-row book leaves its groups out when it is built for a forward pass that
+        is known to go by rows and no gradient is being recorded (they are built on demand later:
+        :meth:`grouped`)."""
         rows = self.in_rows if transposed else self.out_rows
-        buf = _Buffers(rows, self.kv, self.z_ptr.device, self._pairs_per_row(transposed) >= BY_ROW_MIN_PAIRS)
+        by_row = self._pairs_per_row(transposed) >= BY_ROW_MIN_PAIRS
+        if groups is None:
+            groups = not (by_row and weight is not None and not torch.is_grad_enabled()
+                          and weight.dim() == 3 and self._rows_kernel_takes(weight, weight_transposed))
+        buf = _Buffers(rows, self.kv, self.z_ptr.device, by_row, groups)
         g, b = self.geom(), buf.struct()
         lib = L.lib()
         if weight is None:
@@ -237,6 +261,18 @@ class RuleBook:
         return buf
 
     # -- views ------------------------------------------------------------
+    def grouped(self, transposed: bool = False) -> _Buffers:
+        """The forward (or transposed) book with its groups, which wgrad, the padded tensors and the
+        grouped convolution kernels need; rebuilt once if it was made for a by-row forward pass only."""
+        buf = self.transposed() if transposed else self.fwd
+        if not buf.groups:
+            buf = self._build(transposed, groups=True)
+            if transposed:
+                self._bwd = buf
+            else:
+                self.fwd = buf
+        return buf
+
     def transposed(self) -> _Buffers:
         """Book stationary on input rows (what dgrad gathers through)."""
         if self._bwd is None:
@@ -256,7 +292,7 @@ class RuleBook:
         key = (int(tile_size[0]), int(tile_size[1]))
         if key not in self._padded:
             lib = L.lib()
-            g, b = self.geom(), self.fwd.struct()
+            g, b = self.geom(), self.grouped().struct()
             dev = self.z_ptr.device
             ntile = lib.sph_num_tiles(C.byref(g), *key)
             nbr = torch.empty(max(self.out_rows, 1) * self.kv, dtype=torch.int32, device=dev)

@@ -212,7 +212,21 @@ def rule_conv(feature: torch.Tensor, weight: torch.Tensor, rules, ruleSize, outN
                                                            weight.shape[1], weight.shape[2]):
         raise L.SphconvError("packed weight of %d bytes does not belong to a weight of shape %s"
                              % (packed.numel(), tuple(weight.shape)))
-    return _apply(feature, packed, weight.shape[1], weight.shape[2], book.fwd, scale, shift, relu)
+    return _apply(feature, packed, weight.shape[1], weight.shape[2], _conv_buffers(book, feature, weight, False),
+                  scale, shift, relu)
+
+
+def _conv_buffers(book, feature, weight, transposed: bool):
+    """The book's buffers for one convolution call; a book kept by rows only gets its groups built
+    when this call cannot go by rows."""
+    buf = book.transposed() if transposed else book.fwd
+    if buf.groups:
+        return buf
+    es = feature.element_size()
+    kdim, ndim = weight.shape[1], weight.shape[2]
+    by_rows = (kdim * es) % 16 == 0 and kdim * es <= 128 and (ndim * es) % 16 == 0 and feature.data_ptr() % 16 == 0 \
+        and feature.shape[0] > 0
+    return buf if by_rows else book.grouped(transposed)
 
 
 def rule_conv_int8(feature: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, rules, ruleSize,
@@ -224,7 +238,7 @@ def rule_conv_int8(feature: torch.Tensor, weight: torch.Tensor, scale: torch.Ten
     _check_conv_args(feature, weight)
     book = _as_book(rules, ruleSize, feature.shape[0], int(outNNZ))
     packed = _packed_weight(weight, False)
-    return _apply(feature, packed, weight.shape[1], weight.shape[2], book.fwd,
+    return _apply(feature, packed, weight.shape[1], weight.shape[2], _conv_buffers(book, feature, weight, False),
                   scale.to(torch.float32).contiguous())
 
 
@@ -236,7 +250,7 @@ def rule_conv_d_feature(feature: torch.Tensor, weight: torch.Tensor, rules, rule
     weight = _check_conv_args(feature, weight)
     book = _as_book(rules, ruleSize, int(outNNZ), feature.shape[0])
     packed = _packed_weight(weight, False)
-    return _apply(feature, packed, weight.shape[1], weight.shape[2], book.transposed())
+    return _apply(feature, packed, weight.shape[1], weight.shape[2], _conv_buffers(book, feature, weight, True))
 
 
 def rule_conv_d_weight(feature: torch.Tensor, d_featureOut: torch.Tensor, rules, ruleSize) -> torch.Tensor:
@@ -251,7 +265,7 @@ def rule_conv_d_weight(feature: torch.Tensor, d_featureOut: torch.Tensor, rules,
     n = lib.sph_wgrad_partial_elems(book.kv, ic, oc, book.out_rows)
     partial = torch.empty(max(n, 1), dtype=torch.float32, device=feature.device)
     dw = torch.empty((book.kv, ic, oc), dtype=feature.dtype, device=feature.device)
-    b = book.fwd.struct()
+    b = book.grouped().struct()
     L.check(lib.sph_conv_wgrad(L.dtype_code(feature.dtype), L.ptr(feature), feature.shape[0], ic,
                                L.ptr(d_out), oc, C.byref(b), L.ptr(partial), L.ptr(dw), L.stream()))
     return dw

@@ -419,3 +419,41 @@ def test_weight_packed_by_the_rule_launch(dtype, ic, oc, subm):
     assert torch.equal(a, b)
     with pytest.raises(sphconv_amd.SphconvError):
         ext.rule_conv(feat, w, book, None, book.out_rows, packed=packed[:-1024])
+
+
+def test_forward_only_book_builds_its_groups_on_demand(pair_form):
+    """A by-row book made for a forward pass without gradients leaves its groups out; wgrad, the padded
+    tensors and a call that cannot go by rows build them when they are asked for."""
+    from sphconv_amd.rulebook import RuleBook
+    rng = np.random.default_rng(21)
+    B, shape = 2, [6, 10, 8]
+    occ = rng.random((B, *shape)) < 0.5
+    idx = np.argwhere(occ).astype(np.int32)
+    _, z_idx, z_ptr, _ = H.csr_from_indices(idx, B, shape)
+    n = z_idx.shape[0]
+    feat = torch.tensor(rng.standard_normal((n, 32)), dtype=torch.float32).half().to(G.DEV)
+    w = torch.tensor(_weights(rng, 27, 32, 16)).half().to(G.DEV)
+    zi, zp = G.t(z_idx), G.t(z_ptr)
+    ref_book = RuleBook.build_subm(zi, zp, B, shape, [3, 3, 3])
+    want = ext.rule_conv(feat, w, ref_book, None, n)
+    with torch.no_grad():
+        book, packed = RuleBook.build_subm(zi, zp, B, shape, [3, 3, 3], weight=w)
+    assert book.fwd.groups == (pair_form == "groups")
+    assert book.num_pairs() == ref_book.num_pairs()
+    got = ext.rule_conv(feat, w, book, None, n, packed=packed)
+    assert torch.equal(got, want)
+    # 12 fp16 input channels are 24-byte rows: not a by-row call, needs the groups
+    w12 = torch.tensor(_weights(rng, 27, 12, 16)).half().to(G.DEV)
+    f12 = feat[:, :12].contiguous()
+    assert torch.equal(ext.rule_conv(f12, w12, book, None, n), ext.rule_conv(f12, w12, ref_book, None, n))
+    assert book.fwd.groups
+    with torch.no_grad():
+        book, _ = RuleBook.build_subm(zi, zp, B, shape, [3, 3, 3], weight=w)
+    g = torch.tensor(rng.standard_normal((n, 16)), dtype=torch.float32).half().to(G.DEV)
+    assert torch.equal(ext.rule_conv_d_weight(feat, g, book, None), ext.rule_conv_d_weight(feat, g, ref_book, None))
+    assert book.fwd.groups
+    with torch.no_grad():
+        book, _ = RuleBook.build_subm(zi, zp, B, shape, [3, 3, 3], weight=w)
+    r1, s1 = book.padded((2, 2))
+    r2, s2 = ref_book.padded((2, 2))
+    assert torch.equal(s1, s2) and torch.equal(r1, r2)
