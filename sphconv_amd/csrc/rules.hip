@@ -391,34 +391,48 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     // thread first issues the two fiber-bound loads of all its items, then the first
     // three S2 coordinates of every fiber, and only then compares; longer fibers finish
     // in a loop.
+    // kThreads is a multiple of R, so a thread meets the same row in every item: what depends on the row
+    // only is fetched from LDS and multiplied once, and an item costs a handful of integer operations
+    // (k0 = k01 / K1 by a 16-bit reciprocal, exact for the k01 < 256 that a kernel volume <= 128 allows)
+    static_assert(kThreads % R == 0, "a thread's items must share a row");
+    const int my_rl = tid & (R - 1);
+    const bool my_ok = my_rl < nrows && s_col[my_rl] >= 0;
+    const int my_rr = my_ok ? my_rl : 0;
+    const int my_zz = s_z[my_rr];
+    const int my_a0 = TRANSPOSED ? s_c0[my_rr] + a.cv.p0 : s_c0[my_rr] * a.cv.s0 - a.cv.p0;
+    const int my_a1 = TRANSPOSED ? s_c1[my_rr] + a.cv.p1 : s_c1[my_rr] * a.cv.s1 - a.cv.p1;
+    const int my_col0 = s_b[my_rr] * a.P.n0;
+    const int my_slot = my_rr * KV;
+    const unsigned inv_k1 = (65536u + a.cv.K1 - 1) / a.cv.K1;
+    const bool unit_stride = a.cv.s0 == 1 && a.cv.s1 == 1;
     for (int base = 0; !by_masks && base < K01 * R; base += kThreads * kJoinItems) {
-        int ps[kJoinItems], len[kJoinItems], slot[kJoinItems], zz[kJoinItems];
+        int ps[kJoinItems], len[kJoinItems], slot[kJoinItems];
         int raw_e[kJoinItems], raw_s[kJoinItems];
         bool ok[kJoinItems];
 #pragma unroll
         for (int j = 0; j < kJoinItems; j++) {
-            const int it = base + j * kThreads + tid;
-            const int rl = it & (R - 1);
-            const int k01 = it / R;
-            ok[j] = it < K01 * R && rl < nrows && s_col[rl] >= 0;
-            const int rr = ok[j] ? rl : 0;
-            const int k0 = k01 / a.cv.K1, k1 = k01 - k0 * a.cv.K1;
+            const int k01 = (base + j * kThreads + tid) / R;
+            ok[j] = k01 < K01 && my_ok;
+            const int k0 = (int)(((unsigned)k01 * inv_k1) >> 16), k1 = k01 - k0 * a.cv.K1;
             int y0, y1;
             if (!TRANSPOSED) {
-                y0 = s_c0[rr] * a.cv.s0 - a.cv.p0 + k0;
-                y1 = s_c1[rr] * a.cv.s1 - a.cv.p1 + k1;
+                y0 = my_a0 + k0;
+                y1 = my_a1 + k1;
             } else {
-                int t0 = s_c0[rr] + a.cv.p0 - k0, t1 = s_c1[rr] + a.cv.p1 - k1;
-                if (t0 < 0 || t1 < 0 || t0 % a.cv.s0 || t1 % a.cv.s1) ok[j] = false;
-                y0 = t0 / a.cv.s0;
-                y1 = t1 / a.cv.s1;
+                y0 = my_a0 - k0;
+                y1 = my_a1 - k1;
+                if (y0 < 0 || y1 < 0) ok[j] = false;
+                if (!unit_stride) { // uniform branch: divisions only for strided layers
+                    if (y0 % a.cv.s0 || y1 % a.cv.s1) ok[j] = false;
+                    y0 /= a.cv.s0;
+                    y1 /= a.cv.s1;
+                }
             }
             if (y0 < 0 || y0 >= a.P.n0 || y1 < 0 || y1 >= a.P.n1) ok[j] = false;
-            const int pc = ok[j] ? (s_b[rr] * a.P.n0 + y0) * a.P.n1 + y1 : 0;
+            const int pc = ok[j] ? (my_col0 + y0) * a.P.n1 + y1 : 0;
             raw_e[j] = a.p_ptr[pc];
             raw_s[j] = pc ? a.p_ptr[pc - 1] : 0;
-            slot[j] = rr * KV + k01 * a.cv.K2;
-            zz[j] = s_z[rr];
+            slot[j] = my_slot + k01 * a.cv.K2;
         }
         int z0[kJoinItems], z1[kJoinItems], z2[kJoinItems];
 #pragma unroll
@@ -437,7 +451,7 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
             // k2 of a gathered-side entry with S2 coordinate v: forward v is an input
             // coordinate (k2 = v - (z*s2 - p2)), transposed v is an output coordinate
             // (k2 = z + p2 - v*s2)
-            const int off = TRANSPOSED ? zz[j] + a.cv.p2 : -(zz[j] * a.cv.s2 - a.cv.p2);
+            const int off = TRANSPOSED ? my_zz + a.cv.p2 : -(my_zz * a.cv.s2 - a.cv.p2);
             const int mul = TRANSPOSED ? -a.cv.s2 : 1;
             if (len[j] > 0) { int k2 = off + mul * z0[j]; if (k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j]; }
             if (len[j] > 1) { int k2 = off + mul * z1[j]; if (k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j] + 1; }
