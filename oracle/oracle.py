@@ -386,6 +386,35 @@ def points_to_voxel_v2(points, coors_range, sphere_coors_range, max_points=1, ma
     return voxelize_cells(points, sp, coor, ok, max_points, max_voxels, append_mode)
 
 
+def points_to_voxel_sphere(points, voxel_size, sphere_coors_range, max_points=1, max_voxels=30000):
+    """sphconv/utils/voxelize.py:184-206 -> points_to_voxel_3d_sphere_np (include/point2voxel.h:316-399),
+    the branch without a resolution: ``voxel_size`` (log r, degrees, degrees) and ``sphere_coors_range``
+    (radial bounds in the units of log r, degrees, degrees) -> radians; grid = round(range / voxel size)
+    (:337-340); per point theta = acos(z/r), phi = asin(y/sqrt(x^2+y^2)), log r (:349-366), all float32;
+    coordinates are (theta, phi, r) bins; then the same sequential loop (:370-392)."""
+    f32 = np.float32
+    vs = [f32(voxel_size[0]), f32(np.radians(voxel_size[1])), f32(np.radians(voxel_size[2]))]
+    s = [float(v) for v in sphere_coors_range]
+    rng = np.array([s[0], np.radians(s[1]), np.radians(s[2]), s[3], np.radians(s[4]), np.radians(s[5])]).astype(np.float32)
+    grid = [int(np.floor(np.float64(f32(f32(rng[3 + i] - rng[i]) / vs[i])) + 0.5)) for i in range(3)]   # C round()
+    pts = np.ascontiguousarray(points, dtype=np.float32)
+    x, y, z = pts[:, 0], pts[:, 1], pts[:, 2]
+    with np.errstate(all="ignore"):
+        x2y2 = x * x + y * y
+        r = np.sqrt(x2y2 + z * z)
+        theta = np.arccos(z / r)
+        phi = np.arcsin(y / np.sqrt(x2y2))
+        fb = np.stack([(theta - rng[2]) / vs[2], (phi - rng[1]) / vs[1], (np.log(r) - rng[0]) / vs[0]], axis=1)
+    fl = np.floor(fb)
+    ok = np.isfinite(fb).all(1)
+    for i, g in enumerate((grid[2], grid[1], grid[0])):
+        ok &= (fl[:, i] >= 0) & (fl[:, i] < g)
+    coor = np.where(ok[:, None], np.nan_to_num(fl, nan=0.0, posinf=0.0, neginf=0.0), 0).astype(np.int64)
+    res = voxelize_cells(points, None, coor, ok, max_points, max_voxels, 0)
+    res["grid_size"] = grid
+    return res
+
+
 def simple_voxel(voxels, num_points, num_input_features=4):
     """SimpleVoxel.forward (sphconv/vfe.py:222-228): mean of a voxel's points."""
     v = np.asarray(voxels, dtype=np.float32)

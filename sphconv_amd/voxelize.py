@@ -33,20 +33,37 @@ def points_to_voxel_v2(points, voxel_size, coors_range, sphere_coors_range, coor
                        max_points=1, max_voxels=30000, pad_output=False,
                        resolution_HWD: Optional[List[int]] = None, coord_system: Optional[str] = None,
                        append_mode: int = 0, cells: Optional[torch.Tensor] = None, return_cells: bool = False):
-    """voxelize.py:126-214 (the branch with a resolution).  ``points`` [N,>=4] float32 (numpy or
+    """voxelize.py:126-214.  ``points`` [N,>=4] float32 (numpy or
     torch) -> dict with ``voxels`` [max_voxels,max_points,W], ``coordinates`` [max_voxels,3] int32,
     ``num_points_per_voxel`` [max_voxels] int32, ``voxel_point_mask`` [max_voxels,max_points,1] (GPU
     tensors, zero beyond ``voxel_num``) and ``voxel_num`` (int; one 4-byte device->host read).
-    ``coor_to_voxelidx`` (the reference's dense scratch map) and ``voxel_size`` are accepted and
-    not used.  ``cells`` [N] int64 overrides the computed cells; ``return_cells`` adds them as
-    ``res["cells"]``."""
+    ``coor_to_voxelidx`` (the reference's dense scratch map) is accepted and not used; ``voxel_size``
+    only without ``resolution_HWD`` (then: log-spherical bins of that size, coordinates (theta, phi, r),
+    and no appended columns are filled: point2voxel.h:387-390 copies the point as it is).
+    ``cells`` [N] int64 overrides the computed cells; ``return_cells`` adds them as ``res["cells"]``."""
+    f32 = np.float32
     if resolution_HWD is None:
-        raise L.SphconvError("points_to_voxel_v2 needs resolution_HWD (bins of the three system coordinates)")
-    coord_system = coord_system or "spherical"
-    rng = system_range(coors_range, sphere_coors_range, coord_system).astype(np.float32)
-    grid = [int(v) for v in resolution_HWD]
-    # float32 voxel sizes, as the reference's float instantiation computes them (point2voxel.h:436-439)
-    vs = [np.float32((rng[3 + i] - rng[i]) / np.float32(grid[i])) for i in range(3)]
+        # voxelize.py:184-206 -> points_to_voxel_3d_sphere_np (point2voxel.h:316-399): bins of (log r,
+        # phi, theta) from a voxel size (metres of log r, degrees, degrees) and sphere_coors_range taken
+        # as it is (degrees -> radians; its radial bounds are used in the units of log r, :366); the
+        # grid is round(range / voxel size) (:337-340), all in the points' float32
+        vsz = np.asarray(voxel_size, dtype=np.float64)
+        srg = np.asarray(sphere_coors_range, dtype=np.float64)
+        vs = [f32(vsz[0]), f32(np.radians(vsz[1])), f32(np.radians(vsz[2]))]
+        rng = np.array([srg[0], np.radians(srg[1]), np.radians(srg[2]), srg[3], np.radians(srg[4]), np.radians(srg[5])],
+                       dtype=np.float64).astype(np.float32)
+        grid = [int(np.floor(np.float64(f32(f32(rng[3 + i] - rng[i]) / vs[i])) + 0.5)) for i in range(3)]
+        if min(grid) <= 0:
+            raise L.SphconvError("voxel size %s leaves no cell in range %s" % (list(vsz), list(srg)))
+        coord_system = "l-spherical"
+        pad_cols, append_mode = (3 if append_mode == 1 else 0), 0
+    else:
+        pad_cols = 0
+        coord_system = coord_system or "spherical"
+        rng = system_range(coors_range, sphere_coors_range, coord_system).astype(np.float32)
+        grid = [int(v) for v in resolution_HWD]
+        # float32 voxel sizes, as the reference's float instantiation computes them (point2voxel.h:436-439)
+        vs = [f32((rng[3 + i] - rng[i]) / f32(grid[i])) for i in range(3)]
     if isinstance(points, np.ndarray):
         points = torch.from_numpy(np.ascontiguousarray(points, dtype=np.float32))
     dev = points.device if points.is_cuda else torch.device("cuda", torch.cuda.current_device())
@@ -73,6 +90,8 @@ def points_to_voxel_v2(points, voxel_size, coors_range, sphere_coors_range, coor
                                         int(append_mode), L.ptr(voxels), L.ptr(mask), L.ptr(coors), L.ptr(num),
                                         L.ptr(voxel_num), L.ptr(cells), L.ptr(cell_out), L.ptr(work), nbytes,
                                         L.stream()))
+    if pad_cols:
+        voxels = torch.nn.functional.pad(voxels, (0, pad_cols))
     res = {"voxels": voxels, "coordinates": coors, "num_points_per_voxel": num,
            "voxel_point_mask": mask.reshape(-1, max_points, 1), "voxel_num": int(voxel_num.item())}
     if return_cells:
@@ -105,7 +124,7 @@ class VoxelGeneratorV3:
     def generate(self, points, max_voxels=None):
         res = points_to_voxel_v2(points, self._voxel_size, self._point_cloud_range, self._point_cloud_sphere_range,
                                  None, self._max_num_points, max_voxels or self._max_voxels,
-                                 resolution_HWD=[int(v) for v in self._grid_size],
+                                 resolution_HWD=self._resolution_HWD,
                                  coord_system=self._coord_system, append_mode=self._append_mode)
         for k, v in res.items():
             if k != "voxel_num":

@@ -96,3 +96,42 @@ def test_voxelization_vfe_feeds_the_convolution():
     x = sphconv.SparseConvTensor(batch["voxels"], shape_dwh, 2, indices=batch["coordinates"])
     y = sphconv.SubMConv3d(4, 8, 3).cuda()(x)
     assert y.feature.shape == (2 * voxels.shape[0], 8) and torch.isfinite(y.feature).all()
+
+
+def test_sphere_branch_without_resolution():
+    """points_to_voxel_v2 without resolution_HWD (voxelize.py:184-206) on the reference's scan against the
+    oracle; the radial bounds are given in log r as the reference's C++ reads them (point2voxel.h:366)."""
+    pts = np.fromfile(KITTI, dtype=np.float32).reshape(-1, 4)
+    vs = [(np.log(70.4) - np.log(6.0)) / 64, 90.0 / 512, 12.5 / 64]
+    srange = [float(np.log(6.0)), -45.0, 87.5, float(np.log(70.4)), 45.0, 100.0]
+    want = O.points_to_voxel_sphere(pts, vs, srange, max_points=3, max_voxels=20000)
+    assert want["grid_size"] == [64, 512, 64]
+    got = points_to_voxel_v2(pts, vs, None, srange, None, max_points=3, max_voxels=20000, return_cells=True)
+    # bins depend on float32 acos / asin / log: points within 1e-3 of a bin boundary may fall either way
+    cells = got["cells"].cpu().numpy()
+    x, y, z = pts[:, 0].astype(np.float64), pts[:, 1].astype(np.float64), pts[:, 2].astype(np.float64)
+    r = np.sqrt(x * x + y * y + z * z)
+    fb = np.stack([(np.log(r) - srange[0]) / vs[0], (np.degrees(np.arcsin(y / np.sqrt(x * x + y * y))) + 45.0) / vs[1],
+                   (np.degrees(np.arccos(z / r)) - 87.5) / vs[2]], 1)
+    near = (np.abs(fb - np.rint(fb)) < 1e-3).any(1)
+    ok = np.isfinite(fb).all(1) & (fb >= 0).all(1) & (fb[:, 0] < 64) & (fb[:, 1] < 512) & (fb[:, 2] < 64)
+    ref_cells = np.where(ok, (np.floor(fb[:, 2]) * 512 + np.floor(fb[:, 1])) * 64 + np.floor(fb[:, 0]), -1).astype(np.int64)
+    assert near.mean() < 0.02 and np.array_equal(cells[~near], ref_cells[~near])
+    if np.array_equal(cells, ref_cells):          # no point changed its bin: the whole result is the oracle's
+        n = want["voxel_num"]
+        assert got["voxel_num"] == n
+        assert np.array_equal(got["coordinates"][:n].cpu().numpy(), want["coordinates"][:n])
+        assert np.array_equal(got["voxels"][:n].cpu().numpy(), want["voxels"][:n])
+        assert np.array_equal(got["num_points_per_voxel"][:n].cpu().numpy(), want["num_points_per_voxel"][:n])
+    # the sequential rules on the GPU's own cells
+    seq = O.voxelize_cells(pts, None, np.stack([cells // (512 * 64), (cells // 64) % 512, cells % 64], 1), cells >= 0, 3, 20000)
+    n = seq["voxel_num"]
+    assert got["voxel_num"] == n and n > 1000
+    assert np.array_equal(got["coordinates"][:n].cpu().numpy(), seq["coordinates"][:n])
+    assert np.array_equal(got["voxels"][:n].cpu().numpy(), seq["voxels"][:n])
+    assert np.array_equal(got["num_points_per_voxel"][:n].cpu().numpy(), seq["num_points_per_voxel"][:n])
+    # the generator class passes its missing resolution through
+    gen = VoxelGeneratorV3(vs, [6, -40, -3, 70.4, 40, 1], srange, 3, 20000)
+    assert gen.grid_size.tolist() == [64, 512, 64]
+    res = gen.generate(pts)
+    assert res["voxels"].shape[0] == n and np.array_equal(res["coordinates"].cpu().numpy(), seq["coordinates"][:n])

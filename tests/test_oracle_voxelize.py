@@ -80,3 +80,36 @@ def test_kitti_scan_invariants_and_mean():
     one = res["num_points_per_voxel"][:m] == 1
     assert np.array_equal(mean[one], res["voxels"][:m][one, 0])
     np.testing.assert_allclose(mean[~one], res["voxels"][:m][~one].mean(1), rtol=1e-6)
+
+
+def test_sphere_branch_without_resolution_closed_form():
+    """oracle.points_to_voxel_sphere (point2voxel.h:316-399): grid = round(range / voxel size); a point at
+    the centre of bin (it, ip, ir) of (theta, phi, log r) gets exactly these coordinates, in that order;
+    points outside any of the three ranges are skipped; the rest is the shared sequential loop."""
+    vs = [0.25, 0.5, 2.0]                         # log r, degrees, degrees
+    srange = [1.0, -45.0, 80.0, 4.0, 45.0, 100.0]  # log r from 1 to 4, phi, theta
+    want_grid = [12, 180, 10]
+    bins = [(0, 0, 0), (9, 179, 11), (3, 90, 5), (3, 90, 5), (7, 12, 2)]
+    pts = []
+    for it, ip, ir in bins:
+        theta = np.radians(80.0 + (it + 0.5) * 2.0)
+        phi = np.radians(-45.0 + (ip + 0.5) * 0.5)
+        r = np.exp(1.0 + (ir + 0.5) * 0.25)
+        pts.append([r * np.sin(theta) * np.cos(phi), r * np.sin(theta) * np.sin(phi), r * np.cos(theta), len(pts)])
+    outside = [[np.exp(0.5), 0.0, 0.0, 9.0],                       # log r below the range
+               [-10.0, 0.1, 0.0, 9.0],                             # x < 0: asin folds phi back, theta = 90 is inside -> kept
+               [10.0 * np.cos(np.radians(60)), 10.0 * np.sin(np.radians(60)), 0.0, 9.0],   # phi = 60 degrees
+               [10.0 * np.sin(np.radians(70)), 0.0, 10.0 * np.cos(np.radians(70)), 9.0]]   # theta = 70 degrees
+    allp = np.array(pts + outside, np.float32)
+    res = O.points_to_voxel_sphere(allp, vs, srange, max_points=2, max_voxels=10)
+    assert res["grid_size"] == want_grid
+    # four distinct cells among the five centred points (the third and fourth share one), plus the folded point
+    assert res["voxel_num"] == 5
+    assert res["coordinates"][:4].tolist() == [list(bins[0]), list(bins[1]), list(bins[2]), list(bins[4])]
+    assert res["num_points_per_voxel"][:5].tolist() == [1, 1, 2, 1, 1]
+    assert np.array_equal(res["voxels"][2], allp[[2, 3]])
+    # the folded point: phi = asin(0.1 / 10.0005) ~ 0.573 degrees -> bin 91, theta 90 -> bin 5, log 10 = 2.3026 -> bin 5
+    assert res["coordinates"][4].tolist() == [5, 91, 5]
+    # rounding of the grid: 2.2 / 0.5 = 4.4 -> 4, 2.3 / 0.5 = 4.6 -> 5, exact halves go away from zero (C round)
+    g = O.points_to_voxel_sphere(allp[:1], [0.5, 0.5, 0.5], [0, 0, 0, 2.2, 2.3, 1.25], 1, 1)["grid_size"]
+    assert g == [4, 5, 3]
