@@ -457,3 +457,44 @@ def test_forward_only_book_builds_its_groups_on_demand(pair_form):
     r1, s1 = book.padded((2, 2))
     r2, s2 = ref_book.padded((2, 2))
     assert torch.equal(s1, s2) and torch.equal(r1, r2)
+
+
+@pytest.mark.parametrize("p,shape,ic,oc,dtype", [(0.5, [24, 96, 16], 32, 32, torch.float16), (1.0, [18, 64, 16], 16, 64, torch.float16),
+                                                 (0.08, [64, 256, 24], 32, 16, torch.float16), (0.5, [24, 96, 16], 16, 16, torch.float32),
+                                                 (0.6, [24, 80, 16], 64, 32, torch.int8)])
+def test_by_row_equals_groups_on_large_grids(monkeypatch, p, shape, ic, oc, dtype):
+    """More than 1024 tiles (one wave per tile in the by-row kernel), dense to sparse, rows of 32 and 64
+    bytes: same pairs, same summation order, so bit-identical to the grouped kernel, forward and dgrad."""
+    from sphconv_amd import rulebook
+    from sphconv_amd.rulebook import RuleBook
+    rng = np.random.default_rng(int(p * 100) + ic)
+    B = 8
+    occ = rng.random((B, *shape)) < p
+    idx = np.argwhere(occ).astype(np.int32)
+    _, z_idx, z_ptr, _ = H.csr_from_indices(idx, B, shape)
+    n = z_idx.shape[0]
+    assert n > 1024 * 128
+    zi, zp = G.t(z_idx), G.t(z_ptr)
+    if dtype == torch.int8:
+        feat = torch.tensor(rng.integers(-128, 128, (n, ic), dtype=np.int8)).to(G.DEV)
+        w = torch.tensor(rng.integers(-128, 128, (27, ic, oc), dtype=np.int8)).to(G.DEV)
+        scale = torch.tensor(((rng.random(oc) + 0.5) / 3000.0).astype(np.float32)).to(G.DEV)
+        run = lambda book: ext.rule_conv_int8(feat, w, scale, book, None, n)
+    else:
+        feat = torch.tensor(rng.standard_normal((n, ic)), dtype=torch.float32).to(dtype).to(G.DEV)
+        w = torch.tensor(_weights(rng, 27, ic, oc)).to(dtype).to(G.DEV)
+        run = lambda book: ext.rule_conv(feat, w, book, None, n)
+    out = {}
+    for form, thr in (("groups", float("inf")), ("by_row", 0.0)):
+        monkeypatch.setattr(rulebook, "BY_ROW_MIN_PAIRS", thr)
+        book = RuleBook.build_subm(zi, zp, B, shape, [3, 3, 3])
+        assert (book.fwd.tile_nbr is not None) == (form == "by_row")
+        out[form] = run(book)
+        if dtype != torch.int8:
+            g = torch.tensor(rng.standard_normal((n, oc)), dtype=torch.float32).to(dtype).to(G.DEV) if form == "groups" else g
+            wt = w.permute(0, 2, 1).contiguous()
+            out[form + "_d"] = ext.rule_conv_d_feature(g, wt, book, None, None, n)
+    assert torch.equal(out["groups"], out["by_row"])
+    assert float(out["groups"].float().abs().mean()) > 0
+    if dtype != torch.int8:
+        assert torch.equal(out["groups_d"], out["by_row_d"])
