@@ -35,8 +35,11 @@ class ConvFunction(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             w = weight if weight.dtype == feature.dtype else weight.to(feature.dtype)
             # contraction over oC with W[k]^T: packed straight from [KV,iC,oC], no permuted copy
-            packed = ext._packed_weight(w, True)
-            d_feature = ext._apply(d_out, packed, w.shape[2], w.shape[1], book.transposed())
+            buf, reverse = ext._dgrad_buffers(book, d_out, w.shape[2], w.shape[1])
+            if buf is None:
+                buf = book.transposed()
+            packed = ext._packed_weight(w, True, reverse)
+            d_feature = ext._apply(d_out, packed, w.shape[2], w.shape[1], buf)
         if ctx.needs_input_grad[1]:
             d_weight = ext.rule_conv_d_weight(feature, d_out, book, None).to(weight.dtype)
         return d_feature, d_weight, None, None, None, None, None

@@ -273,8 +273,15 @@ class RuleBook:
                 self.fwd = buf
         return buf
 
+    def mirrored(self) -> bool:
+        """True if the book is its own transpose up to mirroring the offsets (k <-> KV-1-k): submanifold,
+        stride 1, odd kernel, padding K//2 -- then dgrad runs on the forward book with reversed weights."""
+        return bool(self.subm and self.kernel is not None and self.oz_idx is self.z_idx
+                    and all(k % 2 == 1 for k in self.kernel) and all(s == 1 for s in self.stride)
+                    and all(p == k // 2 for p, k in zip(self.padding, self.kernel)))
+
     def transposed(self) -> _Buffers:
-        """Book stationary on input rows (what dgrad gathers through)."""
+        """Book stationary on input rows (what dgrad gathers through when the book is not mirrored)."""
         if self._bwd is None:
             self._bwd = self._convert(True) if self._from_padded is not None else self._build(True)
         return self._bwd

@@ -23,10 +23,10 @@ from .rulebook import RuleBook
 
 __version__ = "hip-gfx950"
 
-def _packed_weight(weight: torch.Tensor, transpose: bool) -> torch.Tensor:
+def _packed_weight(weight: torch.Tensor, transpose: bool, reverse: bool = False) -> torch.Tensor:
     """weight [KV, a, b] -> fragment-ordered copy for the contraction over ``a``
-    (``transpose``: over ``b``, i.e. with W[k]^T).  Packed on every call: the
-    weight may have been updated in place since the last one."""
+    (``transpose``: over ``b``, i.e. with W[k]^T; ``reverse``: offsets in reverse order, W[KV-1-k]).
+    Packed on every call: the weight may have been updated in place since the last one."""
     lib = L.lib()
     w = weight.detach()
     if not w.is_contiguous():
@@ -39,8 +39,21 @@ def _packed_weight(weight: torch.Tensor, transpose: bool) -> torch.Tensor:
     if nbytes == 0:
         raise L.SphconvError("cannot pack weight of shape %s" % (tuple(w.shape),))
     packed = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
-    L.check(lib.sph_weight_pack(dt, L.ptr(w), kv, kdim, ndim, a * b, skk, sn, L.ptr(packed), L.stream()))
+    first, sk = L.ptr(w), a * b
+    if reverse:                                  # start at the last offset and walk backwards
+        first, sk = first + (kv - 1) * a * b * w.element_size(), -a * b
+    L.check(lib.sph_weight_pack(dt, first, kv, kdim, ndim, sk, skk, sn, L.ptr(packed), L.stream()))
     return packed
+
+
+def _dgrad_buffers(book: RuleBook, d_out: torch.Tensor, kdim: int, ndim: int):
+    """(buffers, reverse) for d_feature = sum d_out[out] @ W[k]^T.  A submanifold book with odd kernels is
+    its own transpose with the offsets mirrored (the pair (k, in=i, out=j) has the twin (KV-1-k, in=j,
+    out=i)): the forward book serves, with the weight's offsets reversed, and no transposed book is built."""
+    if book.mirrored():
+        fake_w = torch.empty((book.kv, kdim, ndim), dtype=d_out.dtype, device="meta")
+        return _conv_buffers(book, d_out, fake_w, False), True
+    return None, False
 
 
 def _as_book(rules, rule_size, in_rows: int, out_rows: int) -> RuleBook:
@@ -249,8 +262,11 @@ def rule_conv_d_feature(feature: torch.Tensor, weight: torch.Tensor, rules, rule
     of input rows; returns d_feature [outNNZ,iC]."""
     weight = _check_conv_args(feature, weight)
     book = _as_book(rules, ruleSize, int(outNNZ), feature.shape[0])
-    packed = _packed_weight(weight, False)
-    return _apply(feature, packed, weight.shape[1], weight.shape[2], _conv_buffers(book, feature, weight, True))
+    buf, reverse = _dgrad_buffers(book, feature, weight.shape[1], weight.shape[2])
+    if buf is None:
+        buf = _conv_buffers(book, feature, weight, True)
+    packed = _packed_weight(weight, False, reverse)
+    return _apply(feature, packed, weight.shape[1], weight.shape[2], buf)
 
 
 def rule_conv_d_weight(feature: torch.Tensor, d_featureOut: torch.Tensor, rules, ruleSize) -> torch.Tensor:
