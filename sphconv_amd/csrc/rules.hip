@@ -224,7 +224,7 @@ constexpr int kJoinItems = 5; // (row, k0, k1) items a thread joins per pass, al
 template <bool TRANSPOSED>
 __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
 {
-    extern __shared__ int32_t s_nbr[]; // [R * KV]
+    extern __shared__ __attribute__((aligned(16))) int32_t s_nbr[]; // [R * KV]
     __shared__ int s_col[R];
     __shared__ int s_b[R], s_c0[R], s_c1[R], s_z[R];
     __shared__ EmitScratch s_emit;
@@ -249,7 +249,7 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     // the tile's own S2 coordinates do not depend on the column search: fetch them first
     const int my_z = (tid < nrows) ? a.q_idx[r0 + tid] : 0;
 
-    for (int i = tid; i < R * KV; i += kThreads) s_nbr[i] = -1;
+    for (int i = tid; i < R * KV / 4; i += kThreads) ((int4 *)s_nbr)[i] = make_int4(-1, -1, -1, -1); // R * KV is a multiple of 4
     for (int i = tid; i < R; i += kThreads) s_col[i] = -1;
     __syncthreads();
 
@@ -480,7 +480,7 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
 __global__ __launch_bounds__(kThreads) void book_from_nbr_kernel(const int32_t *nbr, int rows, int KV,
                                                                  int cap, sph_book book)
 {
-    extern __shared__ int32_t s_nbr[];
+    extern __shared__ __attribute__((aligned(16))) int32_t s_nbr[];
     __shared__ EmitScratch s_emit;
     const int tile = blockIdx.x;
     const int r0 = tile * R;
