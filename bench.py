@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0
 # (seed 0), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script scaled by a
 # 256 MiB copy (factors 2.000 / 1.000); commands and raw values: profiles/bench_headline_subm64_f16.md.
 # None for any other workload.
-MEASURED_TRAFFIC_BYTES = {"conv": 9599 * 1024 * 2 + 11924 * 1024, "rules": 1077 * 1024 * 2 + 3461 * 1024}
+MEASURED_TRAFFIC_BYTES = {"conv": 9595 * 1024 * 2 + 11924 * 1024, "rules": 1067 * 1024 * 2 + 3461 * 1024}
 
 
 def parse():
