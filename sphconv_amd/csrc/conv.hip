@@ -722,6 +722,258 @@ __global__ __launch_bounds__(512) void conv_rows_kernel_split(ConvArgs a, int nw
     conv_rows_body<DT, NS, CT, MASKED, 4>(a, nwtot);
 }
 
+
+// ---------------------------------------------------------------------------
+// By stationary row, gathered rows staged in LDS: rows of up to 64 bytes (one MFMA K step), one wave
+// per tile and all output columns.
+//
+// With one K step a (offset, block) step is two or four MFMAs behind a gather of 16 rows; the plain
+// by-row kernel then waits for its gathers (every one a miss of the vector L1: a tile's 27 offsets ask
+// for each neighbouring row about ten times, with the other waves' traffic in between).  The rows a
+// tile's offsets gather lie close together in the feature array: for 9 consecutive offsets (one
+// value of k0 in a 3x3x3 kernel) they are the tile's own range of rows of one line of the grid, a
+// column more on either side.  So the offsets are taken in phases of 9: the wave finds the range
+// [lo, hi] of rows the phase gathers, brings it to LDS as it lies (direct global -> LDS loads, all in
+// flight at once), rewrites the phase's table as one byte per (offset, row) (place in the window, 255 =
+// no pair), and every step's gather is then one 16-byte LDS read per lane.  A phase whose rows do not
+// fit the window (a tile that straddles two lines of the grid, strided layers with wide footprints)
+// gathers from the feature array as before.  The order of summation per row is the plain kernel's
+// (offsets ascending), so results are bit-identical.  Bounds: the LDS (about 10 cycles per 16-row read
+// and CU) and, per phase, one round trip for the window.
+// ---------------------------------------------------------------------------
+constexpr int kWinPhase = 9;           // offsets per window
+constexpr int kWinBytes = 12 * 1024;   // bytes of feature rows a window holds (192 rows of 64 bytes)
+constexpr int kWinTab = kWinPhase * R; // one byte per (offset, row)
+constexpr int kWinNone = 255;
+
+template <sph_dtype DT, int CT, bool MASKED>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void conv_rows_win_kernel(ConvArgs a, int nwtot)
+{
+    typedef typename Traits<DT>::elem elem;
+    typedef typename Traits<DT>::acc4 acc4;
+    typedef int int2v __attribute__((ext_vector_type(2)));
+    constexpr int NB = R / SPH_GROUP;        // 8 blocks of 16 rows
+    constexpr int HB = 4;                    // blocks per stage
+    constexpr int SPO = NB / HB;             // stages per offset
+    constexpr int TL = kWinPhase * R / 2 / kWave; // int2 table entries per lane and phase
+    constexpr int WR = 3;                    // sets of weight fragments: requested three offsets ahead
+    static_assert(kWinPhase % WR == 0, "the ring must divide a phase");
+    extern __shared__ __attribute__((aligned(16))) char s_mem[];
+    uint8_t *s_tab = (uint8_t *)s_mem;       // [kWinPhase][SPO][16 rows][HB blocks]
+    char *s_win = s_mem + kWinTab;           // the window's rows, as they lie in the feature array
+    int32_t *s_tab32 = (int32_t *)s_win;     // a phase without a window: [kWinPhase][R] rows of the feature array
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int tile = sph_xcd_tile(blockIdx.x, (a.book.rows + R - 1) / R);
+    const int r0 = tile * R;
+    if (r0 >= a.book.rows) return;
+    const int nrows = min(R, a.book.rows - r0);
+    const int KV = a.book.KV;
+    const int rb = a.row_bytes;
+    const int nph = (KV + kWinPhase - 1) / kWinPhase;
+    const char *wlane = a.wp + lane * 16;
+    const long wstep = (long)nwtot * (kWave * 16);
+    const int chunk = lane >> 4;
+    const bool live_chunk = chunk * 16 < rb;
+    const int choff = live_chunk ? chunk * 16 : 0;
+
+    acc4 acc[NB][CT];
+#pragma unroll
+    for (int j = 0; j < NB; j++)
+#pragma unroll
+        for (int c = 0; c < CT; c++) acc[j][c] = acc4{0, 0, 0, 0};
+
+    int2v tn[TL]; // the next phase's table, on its way while this phase is worked through
+    auto load_tab = [&](int ph) {
+        const int phc = min(ph, nph - 1);
+        const int2v *src = (const int2v *)(a.book.tile_nbr + ((long)tile * KV + phc * kWinPhase) * R);
+        const int n2 = min(kWinPhase, KV - phc * kWinPhase) * R / 2;
+#pragma unroll
+        for (int i = 0; i < TL; i++) {
+            const int e = lane + kWave * i;
+            tn[i] = src[e < n2 ? e : 0];
+        }
+    };
+    auto load_w = [&](int k, int4v (&w)[CT]) {
+        const char *wk = wlane + (long)min(k, KV - 1) * wstep;
+#pragma unroll
+        for (int c = 0; c < CT; c++) w[c] = *(const int4v *)(wk + (long)c * (kWave * 16));
+    };
+
+    int4v wr[WR][CT];
+    load_tab(0);
+#pragma unroll
+    for (int i = 0; i < WR; i++) load_w(i, wr[i]);
+    for (int ph = 0; ph < nph; ph++) {
+        const int k0 = ph * kWinPhase;
+        const int nk = min(kWinPhase, KV - k0);
+        // this phase's table: validate, find the range of rows it gathers
+        int2v t[TL];
+        int lo = 0x7fffffff, hi = -1;
+#pragma unroll
+        for (int i = 0; i < TL; i++) {
+            const int e = lane + kWave * i;
+            int2v v = tn[i];
+            const bool in = e < nk * R / 2;
+            v.x = (in && (unsigned)v.x < (unsigned)a.feat_rows) ? v.x : -1;
+            v.y = (in && (unsigned)v.y < (unsigned)a.feat_rows) ? v.y : -1;
+            if (v.x >= 0) { lo = min(lo, v.x); hi = max(hi, v.x); }
+            if (v.y >= 0) { lo = min(lo, v.y); hi = max(hi, v.y); }
+            t[i] = v;
+        }
+        load_tab(ph + 1);
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) {
+            lo = min(lo, __shfl_xor(lo, o, kWave));
+            hi = max(hi, __shfl_xor(hi, o, kWave));
+        }
+        lo = __builtin_amdgcn_readfirstlane(lo);
+        hi = __builtin_amdgcn_readfirstlane(hi);
+        if (hi < 0) { // no pair at these offsets
+#pragma unroll
+            for (int i = 0; i < WR; i++) load_w(k0 + kWinPhase + i, wr[i]);
+            continue;
+        }
+        const bool win = hi - lo < kWinNone && (hi - lo + 1) * rb <= kWinBytes;
+        // direct loads write LDS behind the back of the LDS unit's own queue: the last phase's reads must
+        // have returned before the window is overwritten
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (win) {
+#pragma unroll
+            for (int i = 0; i < TL; i++) {
+                // entries 2e and 2e + 1 of the phase: offset e / 64, row 2e % 128 and the next one (same block)
+                const int e = lane + kWave * i;
+                const int row = (2 * e) & (R - 1), blk = row >> 4, n = row & 15;
+                uint8_t *dst = s_tab + (e >> 6) * R + (blk / HB) * (SPH_GROUP * HB) + n * HB + blk % HB;
+                dst[0] = (uint8_t)(t[i].x >= 0 ? t[i].x - lo : kWinNone);
+                dst[HB] = (uint8_t)(t[i].y >= 0 ? t[i].y - lo : kWinNone);
+            }
+            // lane l of load i fills the 16 bytes at i * 1024 + l * 16 of the window
+            const int nbytes = (hi - lo + 1) * rb;
+            const int nld = (nbytes + kWave * 16 - 1) / (kWave * 16);
+            const char *src = a.feat + (long)lo * rb;
+            for (int i = 0; i < nld; i++) {
+                const char *g = src + min((i * kWave + lane) * 16, nbytes - 16);
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
+                                                 (__attribute__((address_space(3))) void *)(s_win + i * (kWave * 16)), 16, 0, 0);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            // stages (offset, HB blocks): table entries two stages ahead, rows one stage ahead
+            const int ns = nk * SPO;
+            auto tab = [&](int st, int (&id)[HB]) {
+                const int sc = min(st, ns - 1);
+                const uint8_t *p = s_tab + (sc / SPO) * R + (sc % SPO) * (SPH_GROUP * HB) + (lane & 15) * HB;
+                const uint32_t pk = HB == 4 ? *(const uint32_t *)p : *(const uint16_t *)p;
+#pragma unroll
+                for (int j = 0; j < HB; j++) id[j] = (pk >> (8 * j)) & 255;
+            };
+            auto rows = [&](const int (&id)[HB], int4v (&x)[HB]) {
+#pragma unroll
+                for (int j = 0; j < HB; j++) // a slot without a pair reads a row of its own: no two lanes on one bank
+                    x[j] = *(const int4v *)(s_win + (id[j] != kWinNone ? id[j] : (lane & 15)) * rb + choff);
+            };
+            int id1[HB], id2[HB];
+            int4v x1[HB];
+            tab(0, id1);
+            tab(1, id2);
+            rows(id1, x1);
+            for (int k9 = 0; k9 < nk; k9 += WR) {
+#pragma unroll
+                for (int i = 0; i < WR; i++) {
+                    if (k9 + i < nk) {
+#pragma unroll
+                        for (int h = 0; h < SPO; h++) {
+                            const int st = (k9 + i) * SPO + h;
+                            int idc[HB];
+                            int4v xc[HB];
+#pragma unroll
+                            for (int j = 0; j < HB; j++) { idc[j] = id1[j]; xc[j] = x1[j]; id1[j] = id2[j]; }
+                            rows(id1, x1);
+                            tab(st + 2, id2);
+#pragma unroll
+                            for (int j = 0; j < HB; j++) {
+                                bool live = idc[j] != kWinNone;
+                                if constexpr (MASKED) live = live && live_chunk;
+                                const int4v x = live ? xc[j] : int4v{0, 0, 0, 0};
+#pragma unroll
+                                for (int c = 0; c < CT; c++) acc[h * HB + j][c] = mfma_step<DT>(wr[i][c], x, acc[h * HB + j][c]);
+                            }
+                        }
+                    }
+                    load_w(k0 + k9 + i + WR, wr[i]);
+                }
+            }
+        } else {
+            // the rows lie too far apart: gathers from the feature array, one offset at a time
+#pragma unroll
+            for (int i = 0; i < TL; i++) ((int2v *)s_tab32)[lane + kWave * i] = t[i];
+#pragma unroll 1
+            for (int k9 = 0; k9 < nk; k9++) {
+                int4v w[CT];
+                load_w(k0 + k9, w);
+#pragma unroll
+                for (int h = 0; h < SPO; h++) {
+                    int id[HB];
+                    int4v x[HB];
+#pragma unroll
+                    for (int j = 0; j < HB; j++) {
+                        id[j] = s_tab32[k9 * R + (h * HB + j) * SPH_GROUP + (lane & 15)];
+                        x[j] = *(const int4v *)(a.feat + (long)max(id[j], 0) * rb + choff);
+                    }
+#pragma unroll
+                    for (int j = 0; j < HB; j++) {
+                        bool live = id[j] >= 0;
+                        if constexpr (MASKED) live = live && live_chunk;
+                        const int4v y = live ? x[j] : int4v{0, 0, 0, 0};
+#pragma unroll
+                        for (int c = 0; c < CT; c++) acc[h * HB + j][c] = mfma_step<DT>(w[c], y, acc[h * HB + j][c]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < WR; i++) load_w(k0 + kWinPhase + i, wr[i]);
+        }
+    }
+
+    // epilogue: a lane holds four consecutive columns of one row per block and column tile
+    const bool plain = DT != SPH_I8 && !a.scale && !a.shift && !a.relu;
+    const bool relu = DT != SPH_I8 && a.relu;
+    float sc[CT][4], sh[CT][4];
+#pragma unroll
+    for (int c = 0; c < CT; c++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int col = min(c * 16 + (lane >> 4) * 4 + j, a.ndim - 1);
+            sc[c][j] = a.scale ? a.scale[col] : 1.f;
+            sh[c][j] = (DT != SPH_I8 && a.shift) ? a.shift[col] : 0.f;
+        }
+    elem *out = (elem *)a.out + (long)r0 * a.ndim;
+#pragma unroll
+    for (int b = 0; b < NB; b++) {
+        const int row = b * SPH_GROUP + (lane & 15);
+        if (row >= nrows) continue;
+#pragma unroll
+        for (int c = 0; c < CT; c++) {
+            const int col = c * 16 + (lane >> 4) * 4;
+            if (col >= a.ndim) continue;
+            union { elem e[4]; uint32_t w[sizeof(elem)]; } u;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float v = DT == SPH_I8 ? (float)(int)acc[b][c][j] : (float)acc[b][c][j];
+                if (!plain) {
+                    v = v * sc[c][j] + sh[c][j];
+                    if (relu) v = v > 0.f ? v : 0.f;
+                }
+                u.e[j] = to_elem<DT>(v);
+            }
+            uint32_t *dst = (uint32_t *)(out + (long)row * a.ndim + col);
+#pragma unroll
+            for (int q = 0; q < (int)sizeof(elem); q++) dst[q] = u.w[q];
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // wgrad
 // ---------------------------------------------------------------------------
@@ -1216,6 +1468,14 @@ int launch_conv_rows_m(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
     // the table, and for 128-byte rows a wave's exchange buffer (up to 4 chunk sets of 16 rows x 80 bytes)
     const size_t lds = (size_t)a.book.KV * R * sizeof(int32_t) + (NS >= 2 ? (size_t)waves * ws * 4 * SPH_GROUP * 80 : 0);
     const dim3 grid(sph_xcd_grid(ntiles)), block(waves * ws * kWave);
+    if constexpr (NS == 1 && CT <= 2) {
+        // one K step, up to 32 columns: the gathered rows go through an LDS window (with 64 columns the
+        // accumulators leave no registers for that kernel's pipeline)
+        if (ws == 1 && waves == 1) {
+            hipLaunchKernelGGL((conv_rows_win_kernel<DT, CT, MASKED>), grid, dim3(kWave), kWinTab + kWinBytes, st, a, nwtot);
+            return sph_check_launch("sph_conv_apply");
+        }
+    }
     if (ws == 4) hipLaunchKernelGGL((conv_rows_kernel_split<DT, NS, CT, MASKED>), grid, block, lds, st, a, nwtot);
     else if constexpr (CT >= 4) hipLaunchKernelGGL((conv_rows_kernel_w2<DT, NS, CT, MASKED>), grid, block, lds, st, a, nwtot);
     else if constexpr (CT == 2) hipLaunchKernelGGL((conv_rows_kernel_w3<DT, NS, CT, MASKED>), grid, block, lds, st, a, nwtot);
