@@ -734,8 +734,9 @@ __global__ __launch_bounds__(512) void conv_rows_kernel_split(ConvArgs a, int nw
 // value of k0 in a 3x3x3 kernel) they are the tile's own range of rows of one line of the grid, a
 // column more on either side.  So the offsets are taken in phases of 9: the wave finds the range
 // [lo, hi] of rows the phase gathers, brings it to LDS as it lies (direct global -> LDS loads, all in
-// flight at once), rewrites the phase's table as one byte per (offset, row) (place in the window, 255 =
-// no pair), and every step's gather is then one 16-byte LDS read per lane.  A phase whose rows do not
+// flight at once), rewrites the phase's table as one byte per (offset, row) (place in the window; slots
+// without a pair point at a row of zeros behind it), and every step's gather is then one 16-byte LDS read
+// per lane, with nothing to select afterwards.  A phase whose rows do not
 // fit the window (a tile that straddles two lines of the grid, strided layers with wide footprints)
 // gathers from the feature array as before.  The order of summation per row is the plain kernel's
 // (offsets ascending), so results are bit-identical.  Bounds: the LDS (about 10 cycles per 16-row read
@@ -744,7 +745,7 @@ __global__ __launch_bounds__(512) void conv_rows_kernel_split(ConvArgs a, int nw
 constexpr int kWinPhase = 9;           // offsets per window
 constexpr int kWinBytes = 12 * 1024;   // bytes of feature rows a window holds (192 rows of 64 bytes)
 constexpr int kWinTab = kWinPhase * R; // one byte per (offset, row)
-constexpr int kWinNone = 255;
+constexpr int kWinMaxRows = 255;          // most rows a window may hold: a byte names any of them or the row of zeros
 
 template <sph_dtype DT, int CT, bool MASKED>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void conv_rows_win_kernel(ConvArgs a, int nwtot)
@@ -834,7 +835,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void co
             for (int i = 0; i < WR; i++) load_w(k0 + kWinPhase + i, wr[i]);
             continue;
         }
-        const bool win = hi - lo < kWinNone && (hi - lo + 1) * rb <= kWinBytes;
+        // a window holds rows lo..hi and, behind them, one row of zeros that slots without a pair read
+        const int nrow = hi - lo + 1;
+        const bool win = nrow <= kWinMaxRows && nrow * rb <= kWinBytes;
         // direct loads write LDS behind the back of the LDS unit's own queue: the last phase's reads must
         // have returned before the window is overwritten
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -845,11 +848,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void co
                 const int e = lane + kWave * i;
                 const int row = (2 * e) & (R - 1), blk = row >> 4, n = row & 15;
                 uint8_t *dst = s_tab + (e >> 6) * R + (blk / HB) * (SPH_GROUP * HB) + n * HB + blk % HB;
-                dst[0] = (uint8_t)(t[i].x >= 0 ? t[i].x - lo : kWinNone);
-                dst[HB] = (uint8_t)(t[i].y >= 0 ? t[i].y - lo : kWinNone);
+                dst[0] = (uint8_t)(t[i].x >= 0 ? t[i].x - lo : nrow);
+                dst[HB] = (uint8_t)(t[i].y >= 0 ? t[i].y - lo : nrow);
             }
             // lane l of load i fills the 16 bytes at i * 1024 + l * 16 of the window
-            const int nbytes = (hi - lo + 1) * rb;
+            const int nbytes = nrow * rb;
             const int nld = (nbytes + kWave * 16 - 1) / (kWave * 16);
             const char *src = a.feat + (long)lo * rb;
             for (int i = 0; i < nld; i++) {
@@ -858,8 +861,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void co
                                                  (__attribute__((address_space(3))) void *)(s_win + i * (kWave * 16)), 16, 0, 0);
             }
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (lane * 16 < rb) *(int4v *)(s_win + nbytes + lane * 16) = int4v{0, 0, 0, 0}; // behind the loads: their last kilobyte may reach here
             // stages (offset, HB blocks): table entries two stages ahead, rows one stage ahead
-            const int ns = nk * SPO;
+            constexpr int ns = kWinPhase * SPO;
             auto tab = [&](int st, int (&id)[HB]) {
                 const int sc = min(st, ns - 1);
                 const uint8_t *p = s_tab + (sc / SPO) * R + (sc % SPO) * (SPH_GROUP * HB) + (lane & 15) * HB;
@@ -869,40 +873,40 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void co
             };
             auto rows = [&](const int (&id)[HB], int4v (&x)[HB]) {
 #pragma unroll
-                for (int j = 0; j < HB; j++) // a slot without a pair reads a row of its own: no two lanes on one bank
-                    x[j] = *(const int4v *)(s_win + (id[j] != kWinNone ? id[j] : (lane & 15)) * rb + choff);
+                for (int j = 0; j < HB; j++) {
+                    // lanes on 16-byte chunks behind the row's end read zeros too
+                    const int r = (MASKED && !live_chunk) ? nrow : id[j];
+                    x[j] = *(const int4v *)(s_win + (__umul24(r, rb) + choff));
+                }
             };
             int id1[HB], id2[HB];
             int4v x1[HB];
             tab(0, id1);
             tab(1, id2);
             rows(id1, x1);
-            for (int k9 = 0; k9 < nk; k9 += WR) {
+            auto round = [&](int k9) {
 #pragma unroll
                 for (int i = 0; i < WR; i++) {
-                    if (k9 + i < nk) {
 #pragma unroll
-                        for (int h = 0; h < SPO; h++) {
-                            const int st = (k9 + i) * SPO + h;
-                            int idc[HB];
-                            int4v xc[HB];
+                    for (int h = 0; h < SPO; h++) {
+                        const int st = (k9 + i) * SPO + h;
+                        int4v xc[HB];
 #pragma unroll
-                            for (int j = 0; j < HB; j++) { idc[j] = id1[j]; xc[j] = x1[j]; id1[j] = id2[j]; }
-                            rows(id1, x1);
-                            tab(st + 2, id2);
+                        for (int j = 0; j < HB; j++) { xc[j] = x1[j]; id1[j] = id2[j]; }
+                        rows(id1, x1);
+                        tab(st + 2, id2);
 #pragma unroll
-                            for (int j = 0; j < HB; j++) {
-                                bool live = idc[j] != kWinNone;
-                                if constexpr (MASKED) live = live && live_chunk;
-                                const int4v x = live ? xc[j] : int4v{0, 0, 0, 0};
+                        for (int j = 0; j < HB; j++)
 #pragma unroll
-                                for (int c = 0; c < CT; c++) acc[h * HB + j][c] = mfma_step<DT>(wr[i][c], x, acc[h * HB + j][c]);
-                            }
-                        }
+                            for (int c = 0; c < CT; c++) acc[h * HB + j][c] = mfma_step<DT>(wr[i][c], xc[j], acc[h * HB + j][c]);
                     }
                     load_w(k0 + k9 + i + WR, wr[i]);
                 }
-            }
+            };
+            // a whole phase as straight-line code (the compiler then counts the weight loads in flight exactly);
+            // offsets past the kernel's last find a table of empty slots
+#pragma unroll
+            for (int k9 = 0; k9 < kWinPhase; k9 += WR) round(k9);
         } else {
             // the rows lie too far apart: gathers from the feature array, one offset at a time
 #pragma unroll
@@ -1472,7 +1476,7 @@ int launch_conv_rows_m(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
         // one K step, up to 32 columns: the gathered rows go through an LDS window (with 64 columns the
         // accumulators leave no registers for that kernel's pipeline)
         if (ws == 1 && waves == 1) {
-            hipLaunchKernelGGL((conv_rows_win_kernel<DT, CT, MASKED>), grid, dim3(kWave), kWinTab + kWinBytes, st, a, nwtot);
+            hipLaunchKernelGGL((conv_rows_win_kernel<DT, CT, MASKED>), grid, dim3(kWave), kWinTab + kWinBytes + 64, st, a, nwtot);
             return sph_check_launch("sph_conv_apply");
         }
     }
