@@ -503,3 +503,47 @@ def test_by_row_equals_groups_on_large_grids(monkeypatch, p, shape, ic, oc, dtyp
     assert float(out["groups"].float().abs().mean()) > 0
     if dtype != torch.int8:
         assert torch.equal(out["groups_d"], out["by_row_d"])
+
+
+@pytest.mark.parametrize("kernel,stride,padding,ic,oc,dtype", [([3, 3, 3], [2, 2, 2], [1, 1, 1], 32, 32, torch.float16),
+                                                              ([3, 3, 3], [1, 2, 1], [1, 1, 1], 16, 32, torch.bfloat16),
+                                                              ([2, 2, 2], [2, 2, 2], [0, 0, 0], 16, 16, torch.float32)])
+def test_by_row_equals_groups_on_large_strided_grids(monkeypatch, kernel, stride, padding, ic, oc, dtype):
+    """Strided layers with more than 1024 output tiles and 64-byte rows (the by-row kernel that stages the
+    gathered rows in LDS, with footprints that do and do not fit its window, kernel volumes that are and
+    are not a multiple of its phase of 9 offsets): forward on the book and dgrad on the transposed book
+    are bit-identical to the grouped kernels, and the forward result matches the oracle's."""
+    from sphconv_amd import rulebook
+    from sphconv_amd.rulebook import RuleBook
+    rng = np.random.default_rng(ic + oc)
+    B, shape = 4, [32, 512, 32]
+    occ = rng.random((B, *shape)) < 0.3
+    idx = np.argwhere(occ).astype(np.int32)
+    _, z_idx, z_ptr, _ = H.csr_from_indices(idx, B, shape)
+    n = z_idx.shape[0]
+    oshape = H.out_shape_of(shape, kernel, stride, padding)
+    zi, zp = G.t(z_idx), G.t(z_ptr)
+    kv = kernel[0] * kernel[1] * kernel[2]
+    feat = torch.tensor(rng.standard_normal((n, ic)), dtype=torch.float32).to(dtype).to(G.DEV)
+    w = torch.tensor(_weights(rng, kv, ic, oc)).to(dtype).to(G.DEV)
+    wt = w.permute(0, 2, 1).contiguous()
+    out = {}
+    for form, thr in (("groups", float("inf")), ("by_row", 0.0)):
+        monkeypatch.setattr(rulebook, "BY_ROW_MIN_PAIRS", thr)
+        book = RuleBook.build(zi, zp, B, shape, oshape, kernel, stride, padding)
+        m = book.out_rows
+        assert m > 1024 * 128 and n > 1024 * 128
+        assert (book.fwd.tile_nbr is not None) == (form == "by_row")
+        out[form] = ext.rule_conv(feat, w, book, None, m)
+        g = torch.tensor(rng.standard_normal((m, oc)), dtype=torch.float32).to(dtype).to(G.DEV) if form == "groups" else g
+        out[form + "_d"] = ext.rule_conv_d_feature(g, wt, book, None, None, n)
+    assert torch.equal(out["groups"], out["by_row"])
+    assert torch.equal(out["groups_d"], out["by_row_d"])
+    ora = O.get_rules(z_idx, z_ptr, B, shape, oshape, kernel, stride, padding, n_max=512)
+    oz_idx, oz_ptr, rules, rule_size, dropped = ora
+    assert dropped == 0 and oz_idx.shape[0] == m
+    want = O.rule_conv(feat.float().cpu().numpy(), w.float().cpu().numpy(), rules, rule_size, m)
+    got = out["by_row"].float().cpu().numpy()
+    tol = {torch.float16: 2.0 ** -9, torch.bfloat16: 2.0 ** -7, torch.float32: 1e-5}[dtype]
+    assert (np.abs(got - want) <= tol * np.abs(want) + 1e-3).all()
+    assert np.abs(want).mean() > 1e-2
