@@ -85,6 +85,12 @@ class _Buffers:
 # Estimated pairs per stationary row from which a book also keeps its pairs by row (and the
 # convolution walks that form).  float("inf") never does, 0 always.
 BY_ROW_MIN_PAIRS = 10.0
+# A book built for a forward pass that is known to go by rows, with no gradient being recorded, leaves
+# its groups out (a fifth of the bytes the rule kernel writes), which moves the break-even down:
+# measured on a 4x32x1024x32 grid, rules + convolution, by rows against by groups: 153/155 us at an
+# estimate of 5.4 pairs per row, 177/205 at 6.75, 215/285 at 8.1 (32->32 fp16); 358/325, 432/460,
+# 502/598 (64->64).  The threshold of such books is this fraction of the one above.
+BY_ROW_FORWARD_ONLY = 0.65
 
 
 class RuleBook:
@@ -141,10 +147,14 @@ class RuleBook:
         is known to go by rows and no gradient is being recorded (they are built on demand later:
         :meth:`grouped`)."""
         rows = self.in_rows if transposed else self.out_rows
-        by_row = self._pairs_per_row(transposed) >= BY_ROW_MIN_PAIRS
+        est = self._pairs_per_row(transposed)
+        by_row = est >= BY_ROW_MIN_PAIRS
         if groups is None:
-            groups = not (by_row and weight is not None and not torch.is_grad_enabled()
-                          and weight.dim() == 3 and self._rows_kernel_takes(weight, weight_transposed))
+            forward_only = (weight is not None and not torch.is_grad_enabled() and weight.dim() == 3
+                            and self._rows_kernel_takes(weight, weight_transposed))
+            if forward_only:
+                by_row = est >= BY_ROW_MIN_PAIRS * BY_ROW_FORWARD_ONLY
+            groups = not (by_row and forward_only)
         buf = _Buffers(rows, self.kv, self.z_ptr.device, by_row, groups)
         g, b = self.geom(), buf.struct()
         lib = L.lib()

@@ -547,3 +547,38 @@ def test_by_row_equals_groups_on_large_strided_grids(monkeypatch, kernel, stride
     tol = {torch.float16: 2.0 ** -9, torch.bfloat16: 2.0 ** -7, torch.float32: 1e-5}[dtype]
     assert (np.abs(got - want) <= tol * np.abs(want) + 1e-3).all()
     assert np.abs(want).mean() > 1e-2
+
+
+def test_forward_only_books_go_by_rows_from_a_lower_density(monkeypatch):
+    """A book built with its layer's weight while no gradient is recorded leaves its groups out, so it keeps
+    the pairs by row from 0.65 x the usual estimate of pairs per row; any other book of the same tensor
+    stays grouped below the usual threshold.  Same results either way."""
+    from sphconv_amd import rulebook
+    from sphconv_amd.rulebook import RuleBook
+    monkeypatch.setattr(rulebook, "BY_ROW_MIN_PAIRS", 10.0)
+    rng = np.random.default_rng(77)
+    B, shape = 2, [16, 64, 16]
+    occ = rng.random((B, *shape)) < 0.3          # estimate 27 * 0.3 = 8.1 pairs per row
+    idx = np.argwhere(occ).astype(np.int32)
+    _, z_idx, z_ptr, _ = H.csr_from_indices(idx, B, shape)
+    n = z_idx.shape[0]
+    zi, zp = G.t(z_idx), G.t(z_ptr)
+    feat = torch.tensor(rng.standard_normal((n, 32)), dtype=torch.float32).half().to(G.DEV)
+    w = torch.tensor(_weights(rng, 27, 32, 32)).half().to(G.DEV)
+    with torch.no_grad():
+        fwd_only, packed = RuleBook.build_subm(zi, zp, B, shape, [3, 3, 3], weight=w)
+    assert 10.0 * rulebook.BY_ROW_FORWARD_ONLY <= fwd_only._pairs_per_row(False) < 10.0
+    assert fwd_only.fwd.tile_nbr is not None and not fwd_only.fwd.groups
+    with torch.enable_grad():
+        training, _ = RuleBook.build_subm(zi, zp, B, shape, [3, 3, 3], weight=w)
+    plain = RuleBook.build_subm(zi, zp, B, shape, [3, 3, 3])
+    for book in (training, plain):
+        assert book.fwd.tile_nbr is None and book.fwd.groups
+    a = ext.rule_conv(feat, w, fwd_only, None, n, packed=packed)
+    b = ext.rule_conv(feat, w, plain, None, n)
+    assert torch.equal(a, b) and float(a.float().abs().mean()) > 0
+    sparse = rng.random((B, *shape)) < 0.2       # estimate 5.4: below both thresholds
+    _, z_idx2, z_ptr2, _ = H.csr_from_indices(np.argwhere(sparse).astype(np.int32), B, shape)
+    with torch.no_grad():
+        book, _ = RuleBook.build_subm(G.t(z_idx2), G.t(z_ptr2), B, shape, [3, 3, 3], weight=w)
+    assert book.fwd.tile_nbr is None and book.fwd.groups
