@@ -91,7 +91,7 @@ typedef struct sph_book {
      * (every offset of every block of 16 rows costs one step, whatever it holds: the faster
      * way from about ten pairs per row upwards).  Null: not kept.
      * A book that keeps this table may leave grp_k, grp_gather and grp_owner null (all three):
-     * the rule kernel then writes only the counts and the table, sph_conv_apply serves the calls
+     * the rule kernel then writes only the table (tile_ngrp and tile_koff stay as they were), sph_conv_apply serves the calls
      * it can walk by rows (rows of 16-byte multiples up to 128 bytes) and refuses the others,
      * sph_conv_wgrad and sph_rules_to_padded_count refuse the book. */
     int32_t *tile_nbr;

@@ -130,6 +130,7 @@ __device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int t
             dst[i] = r < nrows ? nbr[r * KV + k] : -1;
         }
     }
+    if (!book.grp_gather) return; // the caller keeps the pairs by row only: no groups, and no group counts either
 
     for (int k = wave; k < KV; k += kWaves) {
         int r_lo = lane, r_hi = kWave + lane;
@@ -169,7 +170,6 @@ __device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int t
 
     for (int k = tid; k <= KV; k += kThreads)
         book.tile_koff[(long)tile * (KV + 1) + k] = (uint16_t)sc.goff[k];
-    if (!book.grp_gather) return; // the caller keeps the pairs by row only: counts are written, groups are not
     const int ngrp = sc.goff[KV];
     const long gbase_tile = (long)tile * cap;
     for (int slot = tid; slot < ngrp * SPH_GROUP; slot += kThreads) {
