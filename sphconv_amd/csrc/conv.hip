@@ -728,31 +728,32 @@ __global__ __launch_bounds__(512) void conv_rows_kernel_split(ConvArgs a, int nw
 
 
 // ---------------------------------------------------------------------------
-// By stationary row, gathered rows staged in LDS: rows of up to 64 bytes (one MFMA K step), one wave
-// per tile and all output columns.
+// By stationary row, gathered rows staged in LDS: rows of up to 64 bytes (one MFMA K step), up to 32
+// output columns, one wave per tile.
 //
-// With one K step a (offset, block) step is two or four MFMAs behind a gather of 16 rows; the plain
-// by-row kernel then waits for its gathers (every one a miss of the vector L1: a tile's 27 offsets ask
-// for each neighbouring row about ten times, with the other waves' traffic in between).  The rows a
-// tile's offsets gather lie close together in the feature array: for 9 consecutive offsets (one
-// value of k0 in a 3x3x3 kernel) they are the tile's own range of rows of one line of the grid, a
-// column more on either side.  So the offsets are taken in phases of 9: the wave finds the range
-// [lo, hi] of rows the phase gathers, brings it to LDS as it lies (direct global -> LDS loads, all in
-// flight at once), rewrites the phase's table as one byte per (offset, row) (place in the window; slots
-// without a pair point at a row of zeros behind it), and every step's gather is then one 16-byte LDS read
-// per lane, with nothing to select afterwards.  A phase whose rows do not
-// fit the window (a tile that straddles two lines of the grid, strided layers with wide footprints)
-// gathers from the feature array as before.  The order of summation per row is the plain kernel's
-// (offsets ascending), so results are bit-identical.  Bounds: the LDS (about 10 cycles per 16-row read
-// and CU, against 8 for the step's two MFMAs) and, per phase, one round trip for the window; the
-// registers (accumulators, three offsets of weights, the next table) allow two waves per SIMD.
+// With one K step a (offset, block) step is one or two MFMAs behind a gather of 16 rows; the plain by-row
+// kernel then waits for its gathers (every one a miss of the vector L1: a tile's 27 offsets ask for each
+// neighbouring row about ten times, with the other waves' traffic in between).  The rows a tile's offsets
+// gather lie close together in the feature array: for 9 consecutive offsets (one value of k0 in a 3x3x3
+// kernel) they are the tile's own range of rows of one line of the grid, a column more on either side.
+// So the offsets are taken in phases of 9: the wave finds the range [lo, hi] of rows the phase gathers,
+// brings it to LDS as it lies (direct global -> LDS loads, all in flight at once), rewrites the phase's
+// table as one byte per (offset, row) (place in the window; slots without a pair point at a row of zeros
+// behind it), and every step's gather is then one 16-byte LDS read per lane, with nothing to select
+// afterwards.  A phase whose rows do not fit the window (a tile that straddles two lines of the grid,
+// strided layers with wide footprints) gathers from the feature array instead.  The order of summation
+// per row is the plain kernel's (offsets ascending), so results are bit-identical.  Bounds: the LDS
+// (about 10 cycles per 16-row read and CU, against 8 for the step's two MFMAs) and, per phase, one round
+// trip for the window; the registers (accumulators, three offsets of weights, the next table) allow two
+// waves per SIMD, and with 64 output columns they do not suffice (the compiler spills and the kernel
+// halves its speed), so those layers stay with the plain kernel.
 // Measured, fp16, grid 4x32x1024x32 at 40 % occupancy (1.68 M rows, 10.9 pairs per row): 32->32 178 us
 // against 250 us with gathers from the feature array, 16->32 156 against 210.
 // ---------------------------------------------------------------------------
 constexpr int kWinPhase = 9;           // offsets per window
 constexpr int kWinBytes = 16 * 1024;   // bytes of feature rows a window holds (up to 255 rows)
 constexpr int kWinTab = kWinPhase * R; // one byte per (offset, row)
-constexpr int kWinMaxRows = 255;          // most rows a window may hold: a byte names any of them or the row of zeros
+constexpr int kWinMaxRows = 255;       // most rows of a window: a byte names any of them or the row of zeros
 
 template <sph_dtype DT, int CT, bool MASKED>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void conv_rows_win_kernel(ConvArgs a, int nwtot)
