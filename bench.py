@@ -51,6 +51,10 @@ def parse():
     ap.add_argument("--callers", action="store_true",
                     help="also time the callers either side of the path (init_tensor, to_dense, xyz2RangeVoxel, "
                          "points_to_voxel_v2 + mean VFE) with HIP events; reported under 'callers'")
+    ap.add_argument("--configs", action="store_true",
+                    help="also time every phase (rule book, forward, dgrad, wgrad, transposed book) of the "
+                         "single-layer configurations 1, 2, 3, 5a, 5b and of 8 scans of the headline grid in one "
+                         "launch, one call each through the extension's Python API; reported under 'configs'")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 256 MiB device-to-device copies (a kernel of known HBM traffic, "
@@ -206,6 +210,63 @@ def callers_ms(torch, d, seed, iters):
     return out
 
 
+def configs_ms(torch, seed, iters):
+    """Every phase of the single-layer configurations, one call each through the functions the reference's
+    extension module exports (HIP events around `iters` calls; forward and dgrad include the weight pack,
+    `rules` everything a rule book needs, for the strided layer its output coordinates and the one 4-byte
+    device->host read).  `fwd_GBps` / `fwd_TFLOPs` price the forward's algorithmic bytes and flops."""
+    from sphconv_amd import sphconv_cuda as ext
+    from sphconv_amd.rulebook import RuleBook
+    from sphconv_amd.synth import make_config
+    dev = "cuda:0"
+    out = {}
+
+    def run(name, cfg, ic, oc, dtype, strided=False, batch=None):
+        d = make_config(cfg, seed=seed, batch=batch)
+        shape, B, n = d["spatial_shape"], d["batch"], int(d["z_idx"].shape[0])
+        z_idx, z_ptr = torch.tensor(d["z_idx"], device=dev), torch.tensor(d["z_ptr"], device=dev)
+        torch.manual_seed(seed)
+        if dtype == torch.int8:
+            feat = torch.randint(-20, 20, (n, ic), device=dev, dtype=torch.int8)
+            w = torch.randint(-20, 20, (27, ic, oc), device=dev, dtype=torch.int8)
+        else:
+            feat = torch.randn((n, ic), device=dev).to(dtype)
+            w = (torch.randn((27, ic, oc), device=dev) * (2.0 / (27 * ic)) ** 0.5).to(dtype)
+        if strided:
+            out_shape = [(s + 2 - 3) // 2 + 1 for s in shape]
+            mk = lambda: RuleBook.build(z_idx, z_ptr, B, shape, out_shape, [3, 3, 3], [2, 2, 2], [1, 1, 1])
+        else:
+            mk = lambda: RuleBook.build_subm(z_idx, z_ptr, B, shape, [3, 3, 3])
+        book = mk()
+        m, P, e = book.out_rows, book.num_pairs(), feat.element_size()
+        r = {"in_rows": n, "out_rows": m, "pairs": P, "channels": [ic, oc], "dtype": str(dtype).split(".")[-1],
+             "rules_us": 1e3 * event_ms(mk, iters, torch)}
+        if dtype == torch.int8:
+            sc = torch.full((oc,), 0.01, device=dev)
+            r["fwd_us"] = 1e3 * event_ms(lambda: ext.rule_conv_int8(feat, w, sc, book, None, m), iters, torch)
+        else:
+            r["fwd_us"] = 1e3 * event_ms(lambda: ext.rule_conv(feat, w, book, None, m), iters, torch)
+            d_out = torch.randn((m, oc), device=dev).to(dtype)
+            w_t = w.permute(0, 2, 1).contiguous()
+            book.transposed()
+            r["transposed_rules_us"] = 1e3 * event_ms(lambda: book._build(True), iters, torch)
+            r["dgrad_us"] = 1e3 * event_ms(lambda: ext.rule_conv_d_feature(d_out, w_t, book, None, None, n),
+                                           iters, torch)
+            r["wgrad_us"] = 1e3 * event_ms(lambda: ext.rule_conv_d_weight(feat, d_out, book, None), iters, torch)
+        r["fwd_GBps"] = (n * ic * e + m * oc * e + 27 * ic * oc * e + 8 * P) / r["fwd_us"] / 1e3
+        r["fwd_TFLOPs"] = 2.0 * P * ic * oc / r["fwd_us"] / 1e6
+        out[name] = r
+
+    run("config1_subm_16_16_f32", 1, 16, 16, torch.float32)
+    run("config2_subm_32_32_f16", 2, 32, 32, torch.float16)
+    run("headline_subm_64_64_f16", 2, 64, 64, torch.float16)
+    run("config3_k3s2_32_64_f16_b4", 3, 32, 64, torch.float16, strided=True)
+    run("config5a_subm_64_64_i8_b8", 5, 64, 64, torch.int8)
+    run("config5b_subm_64_64_f16_b8", 5, 64, 64, torch.float16)
+    run("headline_grid_8_scans_subm_64_64_f16", 2, 64, 64, torch.float16, batch=8)
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -338,6 +399,8 @@ def main():
     }
     if args.callers:
         result["callers"] = callers_ms(torch, d, args.seed, 50)
+    if args.configs:
+        result["configs"] = configs_ms(torch, args.seed, 30)
     if args.encoder:
         result["encoder_stack"] = encoder_stack_ms(torch, args.seed, 20)
     if not args.no_cpu_baseline:

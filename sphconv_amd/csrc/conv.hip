@@ -1383,33 +1383,51 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
 
 // dw[k][ci][co] = sum of the written slots of offset k, in slot order.  A slot holds one
 // 64x64 block per (iC,oC) block pair, each in accumulator order of MI x NI tiles (see
-// wgrad_wave_kernel).  A workgroup covers 32 consecutive co of one ci; its 8 groups of 32
-// threads each add every 8th slot, and the 8 sub-sums are added in a fixed order.
+// wgrad_wave_kernel).  A thread owns one 16-byte item of a block (four ci of one co), so the
+// slots are read as they were written; a workgroup covers 32 consecutive items, its 8 groups of
+// 32 threads each add every 8th slot (four loads in flight), and the 8 sub-sums are added in a
+// fixed order.
 template <sph_dtype DT>
 __global__ __launch_bounds__(256) void wgrad_slot_reduce_kernel(const float *partial, const int *flags, int slots_per_k,
-                                                                int iC, int oC, int ni_tiles,
+                                                                int iC, int oC, int mi_tiles, int ni_tiles,
                                                                 typename Traits<DT>::elem *dw)
 {
-    __shared__ float s_sum[8][32];
-    const int k = blockIdx.z, ci = blockIdx.y, co = blockIdx.x * 32 + (threadIdx.x & 31), j = threadIdx.x >> 5;
+    __shared__ float4v s_sum[8][32];
+    const int k = blockIdx.z, b = blockIdx.y, t = threadIdx.x & 31, j = threadIdx.x >> 5;
+    const int q = blockIdx.x * 32 + t;       // 16-byte item of the block, in accumulator order
     const int sbn = (oC + kWsBlock - 1) / kWsBlock, nblk = ((iC + kWsBlock - 1) / kWsBlock) * sbn;
-    const int bi = ci / kWsBlock, bj = co / kWsBlock, li = ci % kWsBlock, lj = co % kWsBlock;
-    // accumulator order inside the block: tile (li/16, lj/16), lane = 16*((li%16)/4) + lj%16, value li%4
-    const int off = (((li >> 4) * ni_tiles + (lj >> 4)) * kWave + (((li & 15) >> 2) << 4) + (lj & 15)) * 4 + (li & 3);
-    const long blk = (long)kWsBlock * kWsBlock;
-    const float *p = partial + ((long)k * slots_per_k * nblk + bi * sbn + bj) * blk + off;
+    const int tile = q >> 6, lane = q & 63;
+    const bool live = tile < mi_tiles * ni_tiles;
+    const long blk = (long)kWsBlock * kWsBlock, step = (long)nblk * blk;
+    const float *p = partial + ((long)k * slots_per_k * nblk + b) * blk + q * 4;
     const int *f = flags + (long)k * slots_per_k;
-    float s = 0.f;
-    if (co < oC)
-        for (int c = j; c < slots_per_k; c += 8)
-            if (f[c]) s += p[(long)c * nblk * blk];
-    s_sum[j][threadIdx.x & 31] = s;
-    __syncthreads();
-    if (j == 0 && co < oC) {
-        float t = 0.f;
+    float4v s = {0.f, 0.f, 0.f, 0.f};
+    if (live)
+        for (int c = j; c < slots_per_k; c += 32) {
+            float4v v[4];
 #pragma unroll
-        for (int q = 0; q < 8; q++) t += s_sum[q][threadIdx.x];
-        dw[((long)k * iC + ci) * oC + co] = (typename Traits<DT>::elem)t;
+            for (int u = 0; u < 4; u++) {
+                const int cc = c + 8 * u;
+                v[u] = float4v{0.f, 0.f, 0.f, 0.f};
+                if (cc < slots_per_k && f[cc]) v[u] = *(const float4v *)(p + cc * step);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) s += v[u];
+        }
+    s_sum[j][t] = s;
+    __syncthreads();
+    if (j == 0 && live) {
+        float4v r = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int g = 0; g < 8; g++) r += s_sum[g][t];
+        // accumulator order inside the block: tile (li/16, lj/16), lane = 16*((li%16)/4) + lj%16, value li%4
+        const int ci = (b / sbn) * kWsBlock + (tile / ni_tiles) * 16 + (lane >> 4) * 4;
+        const int co = (b % sbn) * kWsBlock + (tile % ni_tiles) * 16 + (lane & 15);
+        if (co < oC) {
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+                if (ci + v < iC) dw[((long)k * iC + ci + v) * oC + co] = (typename Traits<DT>::elem)r[v];
+        }
     }
 }
 
@@ -1595,8 +1613,8 @@ int launch_wgrad(const WgradArgs &a0, void *dw, hipStream_t st)
 #undef SPH_WGRAD_CASE
         rc = sph_check_launch("sph_conv_wgrad");
         if (rc) return rc;
-        hipLaunchKernelGGL(wgrad_slot_reduce_kernel<DT>, dim3((unsigned)((a.oC + 31) / 32), a.iC, KV), dim3(256), 0, st,
-                           a.partial, a.flags, a.nchunk * kWsSlices, a.iC, a.oC, ni, (elem *)dw);
+        hipLaunchKernelGGL(wgrad_slot_reduce_kernel<DT>, dim3((unsigned)(mi * ni * 2), sb, KV), dim3(256), 0, st,
+                           a.partial, a.flags, a.nchunk * kWsSlices, a.iC, a.oC, mi, ni, (elem *)dw);
         return sph_check_launch("sph_conv_wgrad(reduce)");
     }
     const WgradArgs &a = a0;
