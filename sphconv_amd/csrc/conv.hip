@@ -1385,7 +1385,7 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
 // 64x64 block per (iC,oC) block pair, each in accumulator order of MI x NI tiles (see
 // wgrad_wave_kernel).  A thread owns one 16-byte item of a block (four ci of one co), so the
 // slots are read as they were written; a workgroup covers 32 consecutive items, its 8 groups of
-// 32 threads each add every 8th slot (four loads in flight), and the 8 sub-sums are added in a
+// 32 threads each add every 8th slot (eight loads in flight), and the 8 sub-sums are added in a
 // fixed order.
 template <sph_dtype DT>
 __global__ __launch_bounds__(256) void wgrad_slot_reduce_kernel(const float *partial, const int *flags, int slots_per_k,
@@ -1403,16 +1403,16 @@ __global__ __launch_bounds__(256) void wgrad_slot_reduce_kernel(const float *par
     const int *f = flags + (long)k * slots_per_k;
     float4v s = {0.f, 0.f, 0.f, 0.f};
     if (live)
-        for (int c = j; c < slots_per_k; c += 32) {
-            float4v v[4];
+        for (int c = j; c < slots_per_k; c += 64) {
+            float4v v[8];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
+            for (int u = 0; u < 8; u++) {
                 const int cc = c + 8 * u;
                 v[u] = float4v{0.f, 0.f, 0.f, 0.f};
                 if (cc < slots_per_k && f[cc]) v[u] = *(const float4v *)(p + cc * step);
             }
 #pragma unroll
-            for (int u = 0; u < 4; u++) s += v[u];
+            for (int u = 0; u < 8; u++) s += v[u];
         }
     s_sum[j][t] = s;
     __syncthreads();
