@@ -363,6 +363,8 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
         }
         __syncthreads();
         by_masks = s_bad == 0 && ncols > 0;
+        const bool pow2_s2 = (a.cv.s2 & (a.cv.s2 - 1)) == 0;
+        const int sh_s2 = __ffs(a.cv.s2) - 1;
         if (by_masks) {
             for (int it = tid; it < K01 * R; it += kThreads) {
                 const int rl = it & (R - 1), k01 = it / R;
@@ -377,8 +379,13 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
                         v = zz * a.cv.s2 - a.cv.p2 + k2;
                     } else {
                         const int t = zz + a.cv.p2 - k2;
-                        if (t < 0 || t % a.cv.s2) continue;
-                        v = t / a.cv.s2;
+                        if (pow2_s2) { // uniform: strides 1, 2, 4, ... need no division
+                            if (t < 0 || (t & (a.cv.s2 - 1))) continue;
+                            v = t >> sh_s2;
+                        } else {
+                            if (t < 0 || t % a.cv.s2) continue;
+                            v = t / a.cv.s2;
+                        }
                     }
                     if ((unsigned)v < 64u && ((m >> v) & 1ull))
                         s_nbr[rl * KV + k01 * a.cv.K2 + k2] = st + __popcll(m & ((1ull << v) - 1ull));
@@ -405,6 +412,8 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     const int my_slot = my_rr * KV;
     const unsigned inv_k1 = (65536u + a.cv.K1 - 1) / a.cv.K1;
     const bool unit_stride = a.cv.s0 == 1 && a.cv.s1 == 1;
+    const bool pow2_stride = (a.cv.s0 & (a.cv.s0 - 1)) == 0 && (a.cv.s1 & (a.cv.s1 - 1)) == 0;
+    const int sh_s0 = __ffs(a.cv.s0) - 1, sh_s1 = __ffs(a.cv.s1) - 1;
     for (int base = 0; !by_masks && base < K01 * R; base += kThreads * kJoinItems) {
         int ps[kJoinItems], len[kJoinItems], slot[kJoinItems];
         int raw_e[kJoinItems], raw_s[kJoinItems];
@@ -422,7 +431,11 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
                 y0 = my_a0 - k0;
                 y1 = my_a1 - k1;
                 if (y0 < 0 || y1 < 0) ok[j] = false;
-                if (!unit_stride) { // uniform branch: divisions only for strided layers
+                if (pow2_stride) { // uniform branches: shifts for strides 1, 2, 4, ..., divisions for the others
+                    if ((y0 & (a.cv.s0 - 1)) || (y1 & (a.cv.s1 - 1))) ok[j] = false;
+                    y0 >>= sh_s0;
+                    y1 >>= sh_s1;
+                } else if (!unit_stride) {
                     if (y0 % a.cv.s0 || y1 % a.cv.s1) ok[j] = false;
                     y0 /= a.cv.s0;
                     y1 /= a.cv.s1;
@@ -510,6 +523,8 @@ __device__ unsigned long long column_mask(const OutArgs &a, int b, int o0, int o
 {
     unsigned long long mask = 0;
     const int K01 = a.cv.K0 * a.cv.K1;
+    const bool pow2 = (a.cv.s2 & (a.cv.s2 - 1)) == 0;
+    const int sh2 = __ffs(a.cv.s2) - 1;
     for (int k01 = part; k01 < K01; k01 += step) {
         const int k0 = k01 / a.cv.K1, k1 = k01 - k0 * a.cv.K1;
         int x0 = o0 * a.cv.s0 - a.cv.p0 + k0;
@@ -518,13 +533,26 @@ __device__ unsigned long long column_mask(const OutArgs &a, int b, int o0, int o
         int pc = (b * a.S.n0 + x0) * a.S.n1 + x1;
         int ps, pe;
         fiber_range(a.z_ptr, pc, a.in_rows, ps, pe);
-        for (int e = ps; e < pe; e++) {
-            int z = a.z_idx[e];
-            for (int k2 = 0; k2 < a.cv.K2; k2++) {
-                int t = z + a.cv.p2 - k2;
-                if (t < 0 || t % a.cv.s2) continue;
-                int o2 = t / a.cv.s2;
-                if (o2 < a.O.n2 && (o2 >> 6) == chunk) mask |= 1ull << (o2 & 63);
+        // four entries of the fiber per round, their loads in flight together
+        for (int e0 = ps; e0 < pe; e0 += 4) {
+            int z[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) z[q] = a.z_idx[min(e0 + q, pe - 1)];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                if (e0 + q >= pe) continue;
+                for (int k2 = 0; k2 < a.cv.K2; k2++) {
+                    int t = z[q] + a.cv.p2 - k2;
+                    int o2;
+                    if (pow2) { // uniform: strides 1, 2, 4, ... need no division
+                        if (t < 0 || (t & (a.cv.s2 - 1))) continue;
+                        o2 = t >> sh2;
+                    } else {
+                        if (t < 0 || t % a.cv.s2) continue;
+                        o2 = t / a.cv.s2;
+                    }
+                    if (o2 < a.O.n2 && (o2 >> 6) == chunk) mask |= 1ull << (o2 & 63);
+                }
             }
         }
     }

@@ -90,6 +90,8 @@ def test_reference_lists(coords, args):
     (False, [2, 2, 2], [2, 2, 2], [0, 0, 0]),
     (False, [3, 3, 3], [1, 1, 1], [0, 0, 0]),
     (False, [4, 4, 4], [3, 2, 1], [2, 1, 0]),
+    (False, [3, 3, 3], [1, 2, 3], [1, 1, 1]),   # a stride along S2 that is no power of two: the division path
+    (False, [3, 3, 5], [4, 4, 4], [1, 1, 2]),
 ])
 def test_random_grids(seed, subm, kernel, stride, padding):
     rng = np.random.default_rng(seed)
