@@ -134,7 +134,8 @@ int sph_rules_build_pack(const int32_t *z_idx, const int32_t *z_ptr, int in_rows
  *  1. sph_outcoords_count: per-column output counts into oz_ptr, their inclusive scan in
  *     place (`scratch`: 8-byte aligned device memory of sph_outcoords_scratch_ints(g) int32,
  *     holding the scan's temporary storage and, when O[2] <= 64, each column's 64-bit mask
- *     of active bins), and the total in *total_dev (device int).
+ *     of active bins), and the total in *total_dev (device int; null: not written, the total is
+ *     the last element of oz_ptr, and the call is one launch shorter).
  *  2. after reading *total_dev: sph_outcoords_fill, given the same scratch and oz_ptr, writes
  *     oz_idx (ascending within a column).
  * sph_outcoords_blocks(g) = ceil(columns / 256), the grid of the fill kernel. */

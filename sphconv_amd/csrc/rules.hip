@@ -879,7 +879,7 @@ SPH_EXPORT int sph_outcoords_count(const int32_t *z_idx, const int32_t *z_ptr, i
                                    int32_t *total_dev, void *stream)
 {
     SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_count: bad geometry");
-    SPH_REQUIRE(z_ptr && oz_ptr && scratch && total_dev && in_rows >= 0 && (in_rows == 0 || z_idx),
+    SPH_REQUIRE(z_ptr && oz_ptr && scratch && in_rows >= 0 && (in_rows == 0 || z_idx),
                 SPH_ERR_ARG, "sph_outcoords_count: null argument");
     SPH_REQUIRE((uintptr_t)scratch % 8 == 0, SPH_ERR_ARG, "sph_outcoords_count: scratch must be 8-byte aligned");
     hipStream_t st = (hipStream_t)stream;
@@ -895,6 +895,7 @@ SPH_EXPORT int sph_outcoords_count(const int32_t *z_idx, const int32_t *z_ptr, i
         sph_set_error("sph_outcoords_count: scan: %s", hipGetErrorString(e));
         return SPH_ERR_LAUNCH;
     }
+    if (!total_dev) return SPH_OK; // the caller reads the last element of oz_ptr itself: one launch less
     hipLaunchKernelGGL(copy_last_kernel, dim3(1), dim3(1), 0, st, (const int32_t *)oz_ptr, ncol, total_dev);
     return sph_check_launch("sph_outcoords_count(total)");
 }

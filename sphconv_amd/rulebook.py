@@ -217,14 +217,13 @@ class RuleBook:
         nblk = lib.sph_outcoords_scratch_ints(C.byref(g))
         if nblk < 0:
             L.check(nblk)
-        nblk += nblk & 1                                      # the total sits behind an even count
         oz_ptr = torch.empty((int(batch), int(out_shape[0]), int(out_shape[1])), dtype=torch.int32, device=dev)
-        scratch = torch.empty(nblk + 1, dtype=torch.int32, device=dev)
-        total = scratch[nblk:]
+        scratch = torch.empty(nblk + (nblk & 1), dtype=torch.int32, device=dev)
         n_in = int(z_idx.shape[0])
+        # no separate total: the inclusive scan's last element is read instead (one launch less)
         L.check(lib.sph_outcoords_count(L.ptr(z_idx), L.ptr(z_ptr), n_in, C.byref(g), L.ptr(oz_ptr),
-                                        L.ptr(scratch), total.data_ptr(), L.stream()))
-        out_rows = int(total.item())
+                                        L.ptr(scratch), None, L.stream()))
+        out_rows = int(oz_ptr.view(-1)[-1].item())
         oz_idx = torch.empty(out_rows, dtype=torch.int32, device=dev)
         L.check(lib.sph_outcoords_fill(L.ptr(z_idx), L.ptr(z_ptr), n_in, C.byref(g), L.ptr(scratch),
                                        L.ptr(oz_ptr), L.ptr(oz_idx), out_rows, L.stream()))

@@ -255,3 +255,31 @@ def test_unsorted_long_fibers_take_the_general_join():
         assert dropped == 0
         assert np.array_equal(G.book_triples(book.fwd), G.oracle_triples(rules, rule_size))
         assert np.array_equal(G.book_triples(book.transposed()), G.oracle_triples(rules, rule_size, swap=True))
+
+
+def test_outcoords_total_is_optional():
+    """sph_outcoords_count writes the output row count to *total_dev when given one and skips that launch
+    when not; either way the count is the last element of the scanned oz_ptr."""
+    import ctypes as C
+    from sphconv_amd import _lib as L
+    rng = np.random.default_rng(5)
+    B, shape, out_shape = 2, [9, 20, 12], [5, 10, 6]
+    idx = np.argwhere(rng.random((B, *shape)) < 0.2).astype(np.int32)
+    _, z_idx, z_ptr, _ = H.csr_from_indices(idx, B, shape)
+    zi, zp = G.t(z_idx), G.t(z_ptr)
+    lib = L.lib()
+    g = L.make_geom(B, shape, out_shape, [3, 3, 3], [2, 2, 2], [1, 1, 1], [1, 1, 1])
+    n = lib.sph_outcoords_scratch_ints(C.byref(g))
+    ptrs = []
+    for with_total in (True, False):
+        oz_ptr = torch.empty((B, out_shape[0], out_shape[1]), dtype=torch.int32, device="cuda:0")
+        scratch = torch.empty(n + (n & 1), dtype=torch.int32, device="cuda:0")
+        total = torch.full((1,), -7, dtype=torch.int32, device="cuda:0")
+        L.check(lib.sph_outcoords_count(L.ptr(zi), L.ptr(zp), int(zi.shape[0]), C.byref(g), L.ptr(oz_ptr),
+                                        L.ptr(scratch), L.ptr(total) if with_total else None, L.stream()))
+        torch.cuda.synchronize()
+        assert int(total.item()) == (int(oz_ptr.view(-1)[-1].item()) if with_total else -7)
+        ptrs.append(oz_ptr.cpu().numpy())
+    assert np.array_equal(ptrs[0], ptrs[1])
+    book = RuleBook.build(zi, zp, B, shape, out_shape, [3, 3, 3], [2, 2, 2], [1, 1, 1])
+    assert np.array_equal(book.oz_ptr.cpu().numpy(), ptrs[0]) and book.out_rows == int(ptrs[0].reshape(-1)[-1])
