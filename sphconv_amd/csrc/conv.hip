@@ -1385,7 +1385,7 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
 // 64x64 block per (iC,oC) block pair, each in accumulator order of MI x NI tiles (see
 // wgrad_wave_kernel).  A thread owns one 16-byte item of a block (four ci of one co), so the
 // slots are read as they were written; a workgroup covers 32 consecutive items, its 8 groups of
-// 32 threads each add every 8th slot (eight loads in flight), and the 8 sub-sums are added in a
+// 32 threads each add every 8th slot (up to sixteen loads in flight), and the 8 sub-sums are added in a
 // fixed order.
 template <sph_dtype DT>
 __global__ __launch_bounds__(256) void wgrad_slot_reduce_kernel(const float *partial, const int *flags, int slots_per_k,
@@ -1393,6 +1393,7 @@ __global__ __launch_bounds__(256) void wgrad_slot_reduce_kernel(const float *par
                                                                 typename Traits<DT>::elem *dw)
 {
     __shared__ float4v s_sum[8][32];
+    __shared__ unsigned long long s_flags[16];
     const int k = blockIdx.z, b = blockIdx.y, t = threadIdx.x & 31, j = threadIdx.x >> 5;
     const int q = blockIdx.x * 32 + t;       // 16-byte item of the block, in accumulator order
     const int sbn = (oC + kWsBlock - 1) / kWsBlock, nblk = ((iC + kWsBlock - 1) / kWsBlock) * sbn;
@@ -1402,18 +1403,34 @@ __global__ __launch_bounds__(256) void wgrad_slot_reduce_kernel(const float *par
     const float *p = partial + ((long)k * slots_per_k * nblk + b) * blk + q * 4;
     const int *f = flags + (long)k * slots_per_k;
     float4v s = {0.f, 0.f, 0.f, 0.f};
-    if (live)
-        for (int c = j; c < slots_per_k; c += 64) {
-            float4v v[8];
+    // The flags of 1024 slots at a time become 16 ballot words in LDS, so that a thread's data loads do not
+    // wait for flag loads: per round a thread takes its 16 candidates of two words (slots j, j+8, ... of each),
+    // the loads of the written ones in flight together, and adds them in slot order.
+    for (int base = 0; base < slots_per_k; base += 1024) {
+        __syncthreads();
 #pragma unroll
-            for (int u = 0; u < 8; u++) {
-                const int cc = c + 8 * u;
+        for (int w = 0; w < 4; w++) {
+            const int c = base + w * 256 + (int)threadIdx.x;
+            const unsigned long long m = __ballot(c < slots_per_k && f[c] != 0);
+            if ((threadIdx.x & (kWave - 1)) == 0) s_flags[w * 4 + (threadIdx.x >> 6)] = m;
+        }
+        __syncthreads();
+        if (!live) continue;
+        const int nwords = min(16, (slots_per_k - base + 63) >> 6);
+        for (int w0 = 0; w0 < nwords; w0 += 2) {
+            const unsigned long long m0 = s_flags[w0] >> j, m1 = w0 + 1 < nwords ? s_flags[w0 + 1] >> j : 0ull;
+            float4v v[16];
+#pragma unroll
+            for (int u = 0; u < 16; u++) {
+                const unsigned long long m = u < 8 ? m0 : m1;
+                const int cc = base + (w0 + (u >> 3)) * 64 + j + 8 * (u & 7);
                 v[u] = float4v{0.f, 0.f, 0.f, 0.f};
-                if (cc < slots_per_k && f[cc]) v[u] = *(const float4v *)(p + cc * step);
+                if ((m >> (8 * (u & 7))) & 1ull) v[u] = *(const float4v *)(p + cc * step);
             }
 #pragma unroll
-            for (int u = 0; u < 8; u++) s += v[u];
+            for (int u = 0; u < 16; u++) s += v[u];
         }
+    }
     s_sum[j][t] = s;
     __syncthreads();
     if (j == 0 && live) {
