@@ -89,12 +89,30 @@ __device__ int block_upper_bound(const int32_t *a, int n, int target, int max_sp
 //           selects the rank-th set bit of the mask and stores -- consecutive
 //           threads store consecutive slots, so the book is written coalesced.
 // ---------------------------------------------------------------------------
+// Lives in dynamic LDS behind the neighbour table, sized by the kernel volume (a 3x3x3 kernel needs 0.9 KB
+// where the largest volume would need 4 KB: one more workgroup per CU).
 struct EmitScratch {
-    unsigned long long mask[SPH_MAX_KV][R / 64];
-    int cnt[SPH_MAX_KV];
-    int goff[SPH_MAX_KV + 1];
-    unsigned char gk[SPH_MAX_KV * (R / SPH_GROUP)];
+    unsigned long long (*mask)[R / 64]; // [KV]
+    int *cnt;                           // [KV]
+    int *goff;                          // [KV + 1]
+    unsigned char *gk;                  // [KV * (R / SPH_GROUP)]
 };
+__host__ __device__ inline size_t emit_scratch_bytes(int KV)
+{
+    const size_t b = (size_t)KV * (R / 64) * sizeof(unsigned long long) + (size_t)KV * sizeof(int) +
+                     (size_t)(KV + 1) * sizeof(int) + (size_t)KV * (R / SPH_GROUP);
+    return (b + 7) & ~(size_t)7;
+}
+// `base` must be 8-byte aligned.
+__device__ __forceinline__ EmitScratch emit_scratch_at(void *base, int KV)
+{
+    EmitScratch sc;
+    sc.mask = (unsigned long long (*)[R / 64])base;
+    sc.cnt = (int *)(sc.mask + KV);
+    sc.goff = sc.cnt + KV;
+    sc.gk = (unsigned char *)(sc.goff + KV + 1);
+    return sc;
+}
 
 // Position of the j-th (0-based) set bit of m; m must have more than j bits set.
 __device__ __forceinline__ int select_bit(unsigned long long m, int j)
@@ -116,7 +134,7 @@ __device__ __forceinline__ int select_bit(unsigned long long m, int j)
 }
 
 __device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int tile, int cap,
-                            EmitScratch &sc, const sph_book &book)
+                            const EmitScratch &sc, const sph_book &book)
 {
     static_assert(R == 128, "the occupancy masks assume 128 rows per tile");
     const int tid = threadIdx.x;
@@ -227,7 +245,6 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     extern __shared__ __attribute__((aligned(16))) int32_t s_nbr[]; // [R * KV]
     __shared__ int s_col[R];
     __shared__ int s_b[R], s_c0[R], s_c1[R], s_z[R];
-    __shared__ EmitScratch s_emit;
     __shared__ int s_tmp, s_flag;
 
     const int tid = threadIdx.x;
@@ -297,7 +314,7 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     // leaves the 64 bins sends the whole tile to the general join below.
     bool by_masks = false;
     if (a.long_fibers) {
-        unsigned long long *s_cmask = (unsigned long long *)(s_nbr + R * KV); // [K01][ncols], ncols <= kMaskCols
+        unsigned long long *s_cmask = (unsigned long long *)((char *)(s_nbr + R * KV) + emit_scratch_bytes(KV)); // [K01][ncols], ncols <= kMaskCols
         int *s_cstart = (int *)(s_cmask + kMaskCols * K01);
         __shared__ int s_cj[R], s_rep[R], s_bad;
         __shared__ unsigned long long s_bal[R / kWave];
@@ -485,7 +502,7 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     __syncthreads();
 
     // 3. compaction
-    emit_groups(s_nbr, nrows, r0, KV, tile, a.cap, s_emit, a.book);
+    emit_groups(s_nbr, nrows, r0, KV, tile, a.cap, emit_scratch_at(s_nbr + R * KV, KV), a.book);
 }
 
 // Book builder from a global neighbour table nbr[rows, KV] (used when the rules
@@ -494,13 +511,25 @@ __global__ __launch_bounds__(kThreads) void book_from_nbr_kernel(const int32_t *
                                                                  int cap, sph_book book)
 {
     extern __shared__ __attribute__((aligned(16))) int32_t s_nbr[];
-    __shared__ EmitScratch s_emit;
     const int tile = blockIdx.x;
     const int r0 = tile * R;
     const int nrows = min(R, rows - r0);
     for (int i = threadIdx.x; i < nrows * KV; i += kThreads) s_nbr[i] = nbr[(long)r0 * KV + i];
     __syncthreads();
-    emit_groups(s_nbr, nrows, r0, KV, tile, cap, s_emit, book);
+    emit_groups(s_nbr, nrows, r0, KV, tile, cap, emit_scratch_at(s_nbr + R * KV, KV), book);
+}
+
+// Kernel volumes above 96 need more than 48 KB of dynamic LDS for the neighbour table.
+template <typename K>
+static int allow_lds(K kernel, size_t bytes, const char *who)
+{
+    if (bytes <= 48 * 1024) return SPH_OK;
+    hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) {
+        sph_set_error("%s: hipFuncSetAttribute(%zu bytes of LDS): %s", who, bytes, hipGetErrorString(e));
+        return SPH_ERR_LAUNCH;
+    }
+    return SPH_OK;
 }
 
 // ---------------------------------------------------------------------------
@@ -795,13 +824,15 @@ static int rules_build(const char *who, const int32_t *z_idx, const int32_t *z_p
         a.pack.total = 0;
     }
     if (a.tile_blocks + pack_blocks == 0) return SPH_OK;
-    size_t lds = (size_t)R * KV * sizeof(int32_t);
+    size_t lds = (size_t)R * KV * sizeof(int32_t) + emit_scratch_bytes(KV);
     // masks pay when a fiber of the gathered side serves several rows: four entries on average
     const long p_cols = (long)a.B * a.P.n0 * a.P.n1;
     const size_t lds_masks = (size_t)kMaskCols * (g->K[0] * g->K[1]) * (sizeof(unsigned long long) + sizeof(int32_t));
     a.long_fibers = a.P.n2 <= 64 && (long)a.p_rows >= 4 * p_cols && lds + lds_masks <= 64 * 1024;
     if (a.long_fibers) lds += lds_masks;
     hipStream_t st = (hipStream_t)stream;
+    int rc = transposed ? allow_lds(build_book_kernel<true>, lds, who) : allow_lds(build_book_kernel<false>, lds, who);
+    if (rc) return rc;
     if (!transposed)
         hipLaunchKernelGGL(build_book_kernel<false>, dim3(a.tile_blocks + pack_blocks), dim3(kThreads), lds, st, a);
     else
@@ -969,7 +1000,10 @@ SPH_EXPORT int sph_rules_from_padded(const int32_t *rules, const int32_t *rule_s
     hipLaunchKernelGGL(nbr_from_padded_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, rules,
                        rule_size, ntile, KV, tile_n_max, in_rows, out_rows, transposed, nbr);
     const int nt = sph_book_tiles(rows);
-    hipLaunchKernelGGL(book_from_nbr_kernel, dim3(nt), dim3(kThreads), (size_t)R * KV * sizeof(int32_t), st,
+    const size_t lds = (size_t)R * KV * sizeof(int32_t) + emit_scratch_bytes(KV);
+    int rc = allow_lds(book_from_nbr_kernel, lds, "sph_rules_from_padded");
+    if (rc) return rc;
+    hipLaunchKernelGGL(book_from_nbr_kernel, dim3(nt), dim3(kThreads), lds, st,
                        nbr, rows, KV, sph_book_cap(KV), *book);
     return sph_check_launch("sph_rules_from_padded");
 }

@@ -92,6 +92,7 @@ def test_reference_lists(coords, args):
     (False, [4, 4, 4], [3, 2, 1], [2, 1, 0]),
     (False, [3, 3, 3], [1, 2, 3], [1, 1, 1]),   # a stride along S2 that is no power of two: the division path
     (False, [3, 3, 5], [4, 4, 4], [1, 1, 2]),
+    (True, [5, 5, 5], [1, 1, 1], [2, 2, 2]),      # kernel volume 125: the neighbour table needs 68 KB of LDS
 ])
 def test_random_grids(seed, subm, kernel, stride, padding):
     rng = np.random.default_rng(seed)
