@@ -1502,7 +1502,12 @@ int launch_conv_wave_ct(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st
     switch (nwtot) { // at most two waves per workgroup (launch bound of the kernel)
     case 1: return launch_conv_wave_m<DT, NS, 1>(a, nwtot, ntiles, st);
     case 2: return launch_conv_wave_m<DT, NS, 2>(a, nwtot, ntiles, st);
-    default: return launch_conv_wave_m<DT, NS, 4>(a, nwtot, ntiles, st);
+    default:
+        // int8 rows are 64 bytes: on a full chip two waves per tile (32 columns each, the rows gathered twice)
+        // are faster (configuration 5a: 50.5 -> 45.5 us); with 128-byte fp16 rows they are slower (123 -> 151 us)
+        if constexpr (DT == SPH_I8)
+            if (ntiles > 1024) return launch_conv_wave_m<DT, NS, 2>(a, nwtot, ntiles, st);
+        return launch_conv_wave_m<DT, NS, 4>(a, nwtot, ntiles, st);
     }
 }
 
