@@ -582,3 +582,36 @@ def test_forward_only_books_go_by_rows_from_a_lower_density(monkeypatch):
     with torch.no_grad():
         book, _ = RuleBook.build_subm(G.t(z_idx2), G.t(z_ptr2), B, shape, [3, 3, 3], weight=w)
     assert book.fwd.tile_nbr is None and book.fwd.groups
+
+
+def test_wgrad_many_slots_equals_sum_over_samples():
+    """Rules never cross batch samples, so d_weight of a batch is the sum of the samples' d_weights.  With 14
+    scans of the configuration-3 grid (2.2 M rows, 17 000 tiles) the slot reduction walks more than 1024
+    partial slots per offset, i.e. more than one pass of its flag words; each sample alone needs 80."""
+    from sphconv_amd.rulebook import RuleBook
+    B = 14
+    d = make_config(3, seed=3, batch=B)
+    shape = d["spatial_shape"]
+    n = int(d["z_idx"].shape[0])
+    assert n > 128 * 64 * 256                       # more than 256 chunks of 64 tiles: > 1024 slots per offset
+    ic = oc = 16
+    gen = torch.Generator(device=G.DEV).manual_seed(9)
+    feat = torch.randn((n, ic), device=G.DEV, generator=gen).half()
+    g = torch.randn((n, oc), device=G.DEV, generator=gen).half()
+    zi, zp = G.t(d["z_idx"]), G.t(d["z_ptr"])
+    book = RuleBook.build_subm(zi, zp, B, shape, [3, 3, 3])
+    whole = ext.rule_conv_d_weight(feat, g, book, None).float()
+    ends = d["z_ptr"].reshape(B, -1)[:, -1].astype(np.int64)
+    starts = np.concatenate([[0], ends[:-1]])
+    parts = torch.zeros_like(whole)
+    pairs = 0
+    for b in range(B):
+        s, e = int(starts[b]), int(ends[b])
+        zp_b = G.t((d["z_ptr"][b:b + 1] - s).astype(np.int32))
+        bk = RuleBook.build_subm(zi[s:e].contiguous(), zp_b, 1, shape, [3, 3, 3])
+        parts += ext.rule_conv_d_weight(feat[s:e].contiguous(), g[s:e].contiguous(), bk, None).float()
+        pairs += bk.num_pairs()
+    assert pairs == book.num_pairs()
+    # every part was rounded to fp16 once, the whole once; the sums run over up to 2.2 M products (centre offset)
+    scale = float(whole.abs().max())
+    assert float((whole - parts).abs().max()) <= 2.0 ** -9 * scale * np.sqrt(B) + 1e-2
