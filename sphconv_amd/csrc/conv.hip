@@ -1180,10 +1180,31 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
     // then stay in that XCD's L2.  The slice index is slowest, so that the first slices --
     // often the only ones with work -- spread over all XCDs and start first.
     const int items = KV * a.nchunk, items_grid = (items + SPH_NUM_XCD - 1) / SPH_NUM_XCD * SPH_NUM_XCD;
-    const int h = blockIdx.x / items_grid;
-    const int u = sph_xcd_tile(blockIdx.x - h * items_grid, items);
-    if (u >= items) return;
-    const int chunk = u / KV, k = u - chunk * KV;
+    int h, chunk, k;
+    if ((int)blockIdx.x < items_grid) {
+        h = 0;
+        const int u = sph_xcd_tile(blockIdx.x, items);
+        if (u >= items) return;
+        chunk = u / KV;
+        k = u - chunk * KV;
+    } else {
+        // later slices: the centre offset's come first (a submanifold book has 8 groups per tile there and
+        // about one elsewhere, so they are usually the only later slices with work and should not queue
+        // behind the empty ones), then the other offsets'
+        const int kc = KV / 2, v = (int)blockIdx.x - items_grid, nc = (kWsSlices - 1) * a.nchunk;
+        if (v < nc) {
+            h = 1 + v / a.nchunk;
+            chunk = v % a.nchunk;
+            k = kc;
+        } else {
+            const int r = v - nc, per = a.nchunk * (KV - 1);
+            if (KV == 1 || r >= (kWsSlices - 1) * per) return;
+            h = 1 + r / per;
+            const int q = r % per, kk = q % (KV - 1);
+            chunk = q / (KV - 1);
+            k = kk + (kk >= kc ? 1 : 0);
+        }
+    }
     const int sbn = (a.oC + kWsBlock - 1) / kWsBlock;
     const int ci0 = (blockIdx.y / sbn) * kWsBlock, co0 = (blockIdx.y % sbn) * kWsBlock;
     const int cA = min(kWsBlock, a.iC - ci0), cG = min(kWsBlock, a.oC - co0);
