@@ -998,6 +998,7 @@ struct WgradArgs {
     int cap, ntiles, nchunk;
     float *partial;
     int *flags;      // wave kernel: one per partial slot, 1 = the slot was written
+    int all_slices;  // wave kernel: every offset has its later slices' workgroups (small grids), not only the centre
     int nslots;
 };
 
@@ -1124,7 +1125,7 @@ __global__ void wgrad_reduce_kernel(const float *partial, int KV, int nchunk, in
 // ---------------------------------------------------------------------------
 constexpr int kWsTiles = 64;   // tiles per chunk (one lane each)
 constexpr int kWsSlice = 64;   // groups per slice
-constexpr int kWsSlices = 4;   // workgroups per (offset, chunk): workgroup h takes slices h, h+4
+constexpr int kWsSlices = 4;   // workgroups per chunk at the centre offset (workgroup h takes slices h, h+4, ...); one elsewhere
 constexpr int kWsBlock = 64;   // channels per block side
 
 typedef short short4v __attribute__((ext_vector_type(4)));
@@ -1188,9 +1189,11 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
         chunk = u / KV;
         k = u - chunk * KV;
     } else {
-        // later slices: the centre offset's come first (a submanifold book has 8 groups per tile there and
-        // about one elsewhere, so they are usually the only later slices with work and should not queue
-        // behind the empty ones), then the other offsets'
+        // Later slices: a submanifold book has 8 groups per tile at the centre offset and about one elsewhere, and
+        // a workgroup without work still costs its dispatch (three quarters of the grid found none when every offset
+        // had four).  So only the centre offset has them, numbered first, and at the other offsets the first
+        // workgroup takes every slice -- unless the grid is small (all_slices): then a dense book's offsets need
+        // their four workgroups each to fill the chip, and they follow the centre's.
         const int kc = KV / 2, v = (int)blockIdx.x - items_grid, nc = (kWsSlices - 1) * a.nchunk;
         if (v < nc) {
             h = 1 + v / a.nchunk;
@@ -1198,13 +1201,14 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
             k = kc;
         } else {
             const int r = v - nc, per = a.nchunk * (KV - 1);
-            if (KV == 1 || r >= (kWsSlices - 1) * per) return;
+            if (!a.all_slices || KV == 1 || r >= (kWsSlices - 1) * per) return;
             h = 1 + r / per;
             const int q = r % per, kk = q % (KV - 1);
             chunk = q / (KV - 1);
             k = kk + (kk >= kc ? 1 : 0);
         }
     }
+    const int slice_step = (a.all_slices || k == KV / 2) ? kWsSlices : 1;
     const int sbn = (a.oC + kWsBlock - 1) / kWsBlock;
     const int ci0 = (blockIdx.y / sbn) * kWsBlock, co0 = (blockIdx.y % sbn) * kWsBlock;
     const int cA = min(kWsBlock, a.iC - ci0), cG = min(kWsBlock, a.oC - co0);
@@ -1225,6 +1229,7 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
         if (lane >= d) incl += v;
     }
     const int total = __shfl(incl, kWave - 1, kWave);
+    if (slice_step == 1 && tid < kWsSlices - 1 && blockIdx.y == 0) a.flags[slot + 1 + tid] = 0; // slots nobody fills
     if (h * kWsSlice >= total) {
         if (tid == 0 && blockIdx.y == 0) a.flags[slot] = 0;
         return;
@@ -1334,7 +1339,7 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
     // The single staging area is safe because LDS operations of a wave execute in order.
     constexpr int NB = kWsSlice / GPB / 4;
     constexpr int DEPTH = 3;
-    for (int s0 = h * kWsSlice; s0 < total; s0 += kWsSlices * kWsSlice) {
+    for (int s0 = h * kWsSlice; s0 < total; s0 += slice_step * kWsSlice) {
         const int s1 = min(total, s0 + kWsSlice);
         const int nbatch = (s1 - s0 + GPB - 1) / GPB;
         const int bases = slot_bases(s0);
@@ -1640,7 +1645,10 @@ int launch_wgrad(const WgradArgs &a0, void *dw, hipStream_t st)
         a.nchunk = wgrad_wave_chunks(a.ntiles);
         a.nslots = KV * a.nchunk * kWsSlices;
         a.flags = (int *)(a.partial + (size_t)a.nslots * sb * kWsBlock * kWsBlock);
-        const dim3 grid(sph_xcd_grid(KV * a.nchunk) * kWsSlices, sb);
+        // later slices for every offset only where the whole grid stays small (measured: a full 4x4x128x4 grid, one
+        // chunk, 15 us with them and 33 us without; 8 chunks 32 against 35 us; from 12 chunks on the shorter grid wins)
+        a.all_slices = KV * a.nchunk * kWsSlices <= 1024;
+        const dim3 grid(sph_xcd_grid(KV * a.nchunk) + (kWsSlices - 1) * a.nchunk * (a.all_slices ? KV : 1), sb);
         const int mi = wgrad_tiles(a.iC), ni = wgrad_tiles(a.oC);
         int rc;
 #define SPH_WGRAD_CASE(M, N)                                                                      \
@@ -1776,6 +1784,9 @@ SPH_EXPORT int sph_conv_wgrad(sph_dtype dt, const void *feature, int in_rows, in
     a.ntiles = sph_book_tiles(fwd_book->rows);
     a.nchunk = wgrad_chunks(a.ntiles);
     a.partial = partial;
+    a.nslots = 0;
+    a.flags = nullptr;
+    a.all_slices = 0;
     hipStream_t st = (hipStream_t)stream;
     switch (dt) {
     case SPH_F32: return launch_wgrad<SPH_F32>(a, d_weight, st);
