@@ -998,6 +998,7 @@ struct WgradArgs {
     int cap, ntiles, nchunk;
     float *partial;
     int *flags;      // wave kernel: one per partial slot, 1 = the slot was written
+    int nslice;      // wave kernel: workgroups per chunk at the centre offset (slices h, h + nslice, ... each)
     int all_slices;  // wave kernel: every offset has its later slices' workgroups (small grids), not only the centre
     int nslots;
 };
@@ -1125,7 +1126,8 @@ __global__ void wgrad_reduce_kernel(const float *partial, int KV, int nchunk, in
 // ---------------------------------------------------------------------------
 constexpr int kWsTiles = 64;   // tiles per chunk (one lane each)
 constexpr int kWsSlice = 64;   // groups per slice
-constexpr int kWsSlices = 4;   // workgroups per chunk at the centre offset (workgroup h takes slices h, h+4, ...); one elsewhere
+constexpr int kWsSlices = 8;   // most workgroups per chunk at the centre offset (workgroup h takes slices h, h + nslice, ...);
+                               // WgradArgs::nslice = 8 on small books, 4 on large ones; one workgroup elsewhere
 constexpr int kWsBlock = 64;   // channels per block side
 
 typedef short short4v __attribute__((ext_vector_type(4)));
@@ -1194,25 +1196,25 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
         // had four).  So only the centre offset has them, numbered first, and at the other offsets the first
         // workgroup takes every slice -- unless the grid is small (all_slices): then a dense book's offsets need
         // their four workgroups each to fill the chip, and they follow the centre's.
-        const int kc = KV / 2, v = (int)blockIdx.x - items_grid, nc = (kWsSlices - 1) * a.nchunk;
+        const int kc = KV / 2, v = (int)blockIdx.x - items_grid, nc = (a.nslice - 1) * a.nchunk;
         if (v < nc) {
             h = 1 + v / a.nchunk;
             chunk = v % a.nchunk;
             k = kc;
         } else {
             const int r = v - nc, per = a.nchunk * (KV - 1);
-            if (!a.all_slices || KV == 1 || r >= (kWsSlices - 1) * per) return;
+            if (!a.all_slices || KV == 1 || r >= (a.nslice - 1) * per) return;
             h = 1 + r / per;
             const int q = r % per, kk = q % (KV - 1);
             chunk = q / (KV - 1);
             k = kk + (kk >= kc ? 1 : 0);
         }
     }
-    const int slice_step = (a.all_slices || k == KV / 2) ? kWsSlices : 1;
+    const int slice_step = (a.all_slices || k == KV / 2) ? a.nslice : 1;
     const int sbn = (a.oC + kWsBlock - 1) / kWsBlock;
     const int ci0 = (blockIdx.y / sbn) * kWsBlock, co0 = (blockIdx.y % sbn) * kWsBlock;
     const int cA = min(kWsBlock, a.iC - ci0), cG = min(kWsBlock, a.oC - co0);
-    const int slot = (k * a.nchunk + chunk) * kWsSlices + h;
+    const int slot = (k * a.nchunk + chunk) * a.nslice + h;
 
     // groups of this offset in the chunk's tiles: lane = tile, prefix sums over the wave
     const int t0 = chunk * kWsTiles;
@@ -1229,7 +1231,7 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
         if (lane >= d) incl += v;
     }
     const int total = __shfl(incl, kWave - 1, kWave);
-    if (slice_step == 1 && tid < kWsSlices - 1 && blockIdx.y == 0) a.flags[slot + 1 + tid] = 0; // slots nobody fills
+    if (slice_step == 1 && tid < a.nslice - 1 && blockIdx.y == 0) a.flags[slot + 1 + tid] = 0; // slots nobody fills
     if (h * kWsSlice >= total) {
         if (tid == 0 && blockIdx.y == 0) a.flags[slot] = 0;
         return;
@@ -1643,12 +1645,16 @@ int launch_wgrad(const WgradArgs &a0, void *dw, hipStream_t st)
         WgradArgs a = a0;
         const int sb = sph_div_up(a.iC, kWsBlock) * sph_div_up(a.oC, kWsBlock);
         a.nchunk = wgrad_wave_chunks(a.ntiles);
-        a.nslots = KV * a.nchunk * kWsSlices;
+        // the centre offset's chain is what a small book's kernel lasts: eight workgroups share it there; on large
+        // books four, which halves the partial blocks to write and add (measured: headline scan 29 -> 23.5 us with
+        // eight, 8 scans 109 -> 115 us)
+        a.nslice = a.nchunk <= 16 ? kWsSlices : kWsSlices / 2;
+        a.nslots = KV * a.nchunk * a.nslice;
         a.flags = (int *)(a.partial + (size_t)a.nslots * sb * kWsBlock * kWsBlock);
         // later slices for every offset only where the whole grid stays small (measured: a full 4x4x128x4 grid, one
         // chunk, 15 us with them and 33 us without; 8 chunks 32 against 35 us; from 12 chunks on the shorter grid wins)
-        a.all_slices = KV * a.nchunk * kWsSlices <= 1024;
-        const dim3 grid(sph_xcd_grid(KV * a.nchunk) + (kWsSlices - 1) * a.nchunk * (a.all_slices ? KV : 1), sb);
+        a.all_slices = KV * a.nchunk * 4 <= 1024;
+        const dim3 grid(sph_xcd_grid(KV * a.nchunk) + (a.nslice - 1) * a.nchunk * (a.all_slices ? KV : 1), sb);
         const int mi = wgrad_tiles(a.iC), ni = wgrad_tiles(a.oC);
         int rc;
 #define SPH_WGRAD_CASE(M, N)                                                                      \
@@ -1665,7 +1671,7 @@ int launch_wgrad(const WgradArgs &a0, void *dw, hipStream_t st)
         rc = sph_check_launch("sph_conv_wgrad");
         if (rc) return rc;
         hipLaunchKernelGGL(wgrad_slot_reduce_kernel<DT>, dim3((unsigned)(mi * ni * 2), sb, KV), dim3(256), 0, st,
-                           a.partial, a.flags, a.nchunk * kWsSlices, a.iC, a.oC, mi, ni, (elem *)dw);
+                           a.partial, a.flags, a.nchunk * a.nslice, a.iC, a.oC, mi, ni, (elem *)dw);
         return sph_check_launch("sph_conv_wgrad(reduce)");
     }
     const WgradArgs &a = a0;
@@ -1787,6 +1793,7 @@ SPH_EXPORT int sph_conv_wgrad(sph_dtype dt, const void *feature, int in_rows, in
     a.nslots = 0;
     a.flags = nullptr;
     a.all_slices = 0;
+    a.nslice = kWsSlices;
     hipStream_t st = (hipStream_t)stream;
     switch (dt) {
     case SPH_F32: return launch_wgrad<SPH_F32>(a, d_weight, st);
