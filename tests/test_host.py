@@ -78,3 +78,11 @@ def test_module_construction_and_init():
     assert utils._triple(3) == (3, 3, 3) and utils._triple([1, 2, 3]) == (1, 2, 3)
     sd = conv.state_dict()
     assert list(sd) == ["weight"]
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The path runs on one GPU; bench.py says so and exits before touching any device."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr and r.stdout == ""
