@@ -153,6 +153,8 @@ def test_int8_forward_exact(ic, oc, subm):
     (True, (3, 3, 3), (1, 1, 1), (1, 1, 1)),
     (False, (3, 3, 3), (2, 2, 2), (1, 1, 1)),
     (False, (2, 2, 1), (1, 1, 1), (0, 0, 0)),
+    (True, (1, 1, 1), (1, 1, 1), (0, 0, 0)),      # one offset: the centre is the only one
+    (True, (5, 5, 5), (1, 1, 1), (2, 2, 2)),      # kernel volume 125
 ])
 def test_fp32_backward(ic, oc, subm, kernel, stride, padding):
     case = _random_case(21 + ic, subm, kernel, stride, padding)
