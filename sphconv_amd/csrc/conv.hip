@@ -1533,8 +1533,9 @@ int launch_conv_wave_ct(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st
     default:
         // int8 rows are 64 bytes: on a full chip two waves per tile (32 columns each, the rows gathered twice)
         // are faster (configuration 5a: 50.5 -> 45.5 us); with 128-byte fp16 rows they are slower (123 -> 151 us)
+        // (up to 64 output columns only: more would be four waves, beyond the kernel's launch bound)
         if constexpr (DT == SPH_I8)
-            if (ntiles > 1024) return launch_conv_wave_m<DT, NS, 2>(a, nwtot, ntiles, st);
+            if (ntiles > 1024 && nwtot <= 4) return launch_conv_wave_m<DT, NS, 2>(a, nwtot, ntiles, st);
         return launch_conv_wave_m<DT, NS, 4>(a, nwtot, ntiles, st);
     }
 }

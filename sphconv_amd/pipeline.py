@@ -20,7 +20,10 @@ class ScanPipeline:
     """``submit(feature, z_idx, z_ptr)`` enqueues rules + forward of one scan on the next
     stream slot and returns ``(out, slot)``; ``out`` [n, oC] is a view of that slot's output
     buffer and is overwritten when the slot comes round again (after ``streams`` submits).
-    Call ``wait(slot)`` (or ``synchronize()``) before reading it on another stream."""
+    Call ``wait(slot)`` (or ``synchronize()``) before reading it on another stream.
+    Lifetime of the inputs: ``submit`` records their use on the slot's stream
+    (``Tensor.record_stream``), so the caller may drop or rebind them as soon as it returns;
+    it must not overwrite them in place before the slot's scan has finished (``wait``)."""
 
     def __init__(self, weight: torch.Tensor, batch: int, shape: Sequence[int], kernel: Sequence[int] = (3, 3, 3),
                  max_voxels: int = 1 << 18, streams: int = 3):
@@ -73,6 +76,11 @@ class ScanPipeline:
         side = self._streams[slot]
         if wait_inputs:
             side.wait_stream(torch.cuda.current_stream())   # the inputs were produced on the caller's stream
+        # the kernels below read the inputs on the slot's stream: tell the caching allocator, so that a caller
+        # who drops or rebinds them right after this call does not get their memory handed out again while
+        # those kernels still run
+        for t in (feature, z_idx, z_ptr):
+            t.record_stream(side)
         st = side.cuda_stream
         book = self._books[slot]
         book._struct.rows = n                                 # the slot's buffers hold up to max_voxels rows

@@ -148,6 +148,26 @@ def test_int8_forward_exact(ic, oc, subm):
     assert want.min() == -128 and want.max() == 127 and (np.abs(want) < 100).mean() > 0.3
 
 
+def test_int8_more_than_64_columns_on_more_than_1024_tiles():
+    """int8 64 -> 128 on more than 131 072 rows: the grouped kernel's two-waves-per-tile form is for up to 64
+    output columns only (more would be four waves per tile, beyond its launch bound); bit-exact."""
+    rng = np.random.default_rng(64128)
+    B, shape = 8, [32, 128, 32]
+    idx = np.argwhere(rng.random((B, *shape)) < 0.14).astype(np.int32)
+    case = G.build_case(idx, B, shape, [3, 3, 3], [1, 1, 1], [1, 1, 1], True)
+    n = case["sidx"].shape[0]
+    assert n > 1024 * 128
+    f8 = rng.integers(-128, 128, (n, 64), dtype=np.int8)
+    w8 = rng.integers(-128, 128, (27, 64, 128), dtype=np.int8)
+    scale = ((rng.random(128) + 0.5) / 3000.0).astype(np.float32)
+    _, _, rules, rule_size, dropped = O.get_rules_subm(case["z_idx"], case["z_ptr"], B, shape, shape, [3, 3, 3],
+                                                       [1, 1, 1], [1, 1, 1], n_max=512)
+    assert dropped == 0
+    want = O.rule_conv_i8(f8, w8, scale, rules, rule_size, n)
+    got = ext.rule_conv_int8(G.t(f8), G.t(w8), G.t(scale), case["book"], None, n).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("ic,oc", [(4, 4), (16, 16), (32, 64), (64, 64), (9, 21)])
 @pytest.mark.parametrize("subm,kernel,stride,padding", [
     (True, (3, 3, 3), (1, 1, 1), (1, 1, 1)),
@@ -335,34 +355,41 @@ def _full_size_case(cfg):
     return d, book, ora
 
 
-@pytest.mark.parametrize("cfg,ic,oc", [(2, 32, 32), (3, 32, 64), (5, 64, 64)])
-def test_configs_full_size_fp16(cfg, ic, oc):
-    """BASELINE configurations 2, 3 and 5b at full size: fp16 storage / fp32 accumulate against
-    the C oracle (fp32) on the same fp16-rounded inputs; 5b also dgrad and wgrad."""
+@pytest.mark.parametrize("cfg,ic,oc,dtype,backward", [
+    (2, 32, 32, torch.float16, False), (3, 32, 64, torch.float16, False), (5, 64, 64, torch.float16, True),
+    (2, 64, 64, torch.float16, True),      # the shape the benchmark times: configuration 2's grid at 64 -> 64
+    (2, 64, 64, torch.bfloat16, True), (3, 32, 64, torch.bfloat16, False)],
+    ids=["cfg2-32-32-f16", "cfg3-32-64-f16", "cfg5b-64-64-f16", "headline-64-64-f16", "headline-64-64-bf16",
+         "cfg3-32-64-bf16"])
+def test_configs_full_size_fp16(cfg, ic, oc, dtype, backward):
+    """BASELINE configurations 2, 3, 5b and the benchmark's shape (configuration 2's grid, 64 -> 64) at full
+    size: fp16 / bf16 storage with fp32 accumulate against the C oracle (fp32) on the same rounded inputs;
+    5b and the benchmark's shape also dgrad and wgrad."""
     d, book, (oz_idx, _, rules, rule_size, _) = _full_size_case(cfg)
     rng = np.random.default_rng(cfg)
     n, m = d["z_idx"].shape[0], oz_idx.shape[0]
-    feat = torch.tensor(rng.standard_normal((n, ic)), dtype=torch.float32).half()
-    w = torch.tensor(_weights(rng, 27, ic, oc)).half()
+    ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7   # one rounding to the storage type
+    feat = torch.tensor(rng.standard_normal((n, ic)), dtype=torch.float32).to(dtype)
+    w = torch.tensor(_weights(rng, 27, ic, oc)).to(dtype)
     out = ext.rule_conv(feat.to(G.DEV), w.to(G.DEV), book, None, m)
-    assert out.dtype == torch.float16 and tuple(out.shape) == (m, oc)
+    assert out.dtype == dtype and tuple(out.shape) == (m, oc)
     want = O.rule_conv(feat.float().numpy(), w.float().numpy(), rules, rule_size, m)
     got = out.float().cpu().numpy()
-    # one rounding to fp16 of an fp32 sum of at most 27*ic products (tolerance of north_star: 1e-2 relative)
-    assert (np.abs(got - want) <= 2.0 ** -10 * np.abs(want) + 1e-3).all()
-    if cfg != 5:
+    # one rounding of an fp32 sum of at most 27*ic products (tolerance of north_star: 1e-2 relative)
+    assert (np.abs(got - want) <= ulp * np.abs(want) + 1e-3).all()
+    if not backward:
         return
-    g = torch.tensor(rng.standard_normal((m, oc)), dtype=torch.float32).half()
+    g = torch.tensor(rng.standard_normal((m, oc)), dtype=torch.float32).to(dtype)
     w_perm = w.permute(0, 2, 1).contiguous()
     d_feat, d_w = ext.rule_conv_backward(g.to(G.DEV), feat.to(G.DEV), w_perm.to(G.DEV), book, None, [1, 1])
     tgs = [-(-d["spatial_shape"][0] // 2), -(-d["spatial_shape"][1] // 2)]
     df_o, dw_o = O.rule_conv_backward(g.float().numpy(), feat.float().numpy(), w_perm.float().numpy(), rules,
                                       rule_size, tgs)
-    assert (np.abs(d_feat.float().cpu().numpy() - df_o) <= 2.0 ** -10 * np.abs(df_o) + 1e-3).all()
+    assert (np.abs(d_feat.float().cpu().numpy() - df_o) <= ulp * np.abs(df_o) + 1e-3).all()
     # d_weight sums ~23 000 products per entry (centre offset: 314 000): fp32 association differs
     # between the oracle and the GPU, both stay within 1e-5 of the sum of absolute products
-    # (E|x||y| = 2/pi for unit normals), plus the rounding to fp16
-    bound = 1e-5 * (2 / np.pi) * rule_size.sum(0)[:, None, None] + 2.0 ** -10 * np.abs(dw_o) + 1e-3
+    # (E|x||y| = 2/pi for unit normals), plus the rounding to the storage type
+    bound = 1e-5 * (2 / np.pi) * rule_size.sum(0)[:, None, None] + ulp * np.abs(dw_o) + 1e-3
     assert (np.abs(d_w.float().cpu().numpy() - dw_o) <= 2 * bound).all()
 
 
