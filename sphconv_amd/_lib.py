@@ -41,7 +41,7 @@ class Epilogue(C.Structure):
 
 
 _lib = None
-ABI_VERSION = 3       # sph_abi_version() of the library these signatures describe
+ABI_VERSION = 4       # sph_abi_version() of the library these signatures describe
 
 _I, _P, _L, _Z = C.c_int, C.c_void_p, C.c_long, C.c_size_t
 _SIGNATURES = {
@@ -56,6 +56,7 @@ _SIGNATURES = {
                                   _L, _P, _P]),
     "sph_outcoords_blocks": (_I, [C.POINTER(Geom)]),
     "sph_outcoords_scratch_ints": (_I, [C.POINTER(Geom)]),
+    "sph_outcoords_state_ints": (_I, [C.POINTER(Geom)]),
     "sph_outcoords_count": (_I, [_P, _P, _I, C.POINTER(Geom), _P, _P, _P, _P]),
     "sph_outcoords_fill": (_I, [_P, _P, _I, C.POINTER(Geom), _P, _P, _P, _I, _P]),
     "sph_rules_to_padded_count": (_I, [C.POINTER(Book), _P, C.POINTER(Geom), _I, _I, _P, _P, _P]),

@@ -2,14 +2,13 @@
 // convolution and the rule book of (kernel offset, gathered row, owner row)
 // triples, replacing the reference's dense [B,S0,S1,S2] position grid and
 // atomic counters (src/sphconv/rules.cu) by fiber joins, wave ballots and
-// prefix popcounts.  All kernels are integer and HBM/latency bound.
+// prefix popcounts; the per-column output counts are scanned inside the kernel
+// that counts them (single pass, decoupled look-back between workgroups).
+// All kernels are integer and HBM/latency bound.
 #include "common.h"
 #include "pack.h"
 
 #include <cstring>
-
-#include <rocprim/device/device_scan.hpp>
-#include <rocprim/functional.hpp>
 
 namespace {
 
@@ -589,7 +588,8 @@ __device__ unsigned long long column_mask(const OutArgs &a, int b, int o0, int o
 }
 
 constexpr int kColLanes = 16;                    // lanes that share one output column
-constexpr int kColsPerBlock = kThreads / kColLanes;
+constexpr int kCountCols = 64;                   // output columns per workgroup of the count kernel
+constexpr int kCountThreads = kCountCols * kColLanes;
 
 // OR over the 16 lanes of a column group (all 16 are active together).
 __device__ __forceinline__ unsigned long long or_reduce16(unsigned long long m)
@@ -603,31 +603,111 @@ __device__ __forceinline__ unsigned long long or_reduce16(unsigned long long m)
     return ((unsigned long long)hi << 32) | lo;
 }
 
-// Per-column counts.  16 lanes share an output column (one input column (k0, k1) each, K0*K1 = 9
-// of them busy for a 3x3x3 kernel), so the fibers that reach a column are walked side by side
-// and small grids still fill the chip.  `masks` (O2 <= 64 only, else null) keeps each column's
-// bin mask for the fill kernel.
-__global__ __launch_bounds__(kThreads) void outcoords_count_kernel(OutArgs a, int32_t *counts,
-                                                                   unsigned long long *masks)
+// State of the scan across workgroups, at the head of the caller's scratch: a ticket counter, a counter
+// of finished workgroups and one 64-bit status word per workgroup (flag in the two top bits, value in
+// the low 32).  All of it is zero between launches: the last workgroup to finish clears it.
+constexpr unsigned long long kScanAggregate = 1ull << 62; // value = sum of the workgroup's own counts
+constexpr unsigned long long kScanInclusive = 2ull << 62; // value = sum of all counts up to and including it
+__host__ __device__ inline int count_blocks(long ncol) { return (int)((ncol + kCountCols - 1) / kCountCols); }
+__host__ __device__ inline long scan_state_ints(long ncol) { return 2 + 2 * (long)count_blocks(ncol); }
+
+__device__ __forceinline__ unsigned long long status_load(const unsigned long long *p)
 {
-    const int ncol = a.B * a.O.n0 * a.O.n1;
-    const int part = threadIdx.x % kColLanes;
-    const int oc = blockIdx.x * kColsPerBlock + threadIdx.x / kColLanes;
-    if (oc >= ncol) return; // whole 16-lane groups leave together
-    const int nchunk = (a.O.n2 + 63) >> 6;
-    const int b = oc / (a.O.n0 * a.O.n1);
-    const int rem = oc - b * (a.O.n0 * a.O.n1);
-    const int o0 = rem / a.O.n1, o1 = rem % a.O.n1;
-    int cnt = 0;
-    for (int ch = 0; ch < nchunk; ch++) {
-        const unsigned long long m = or_reduce16(column_mask(a, b, o0, o1, ch, part, kColLanes));
-        cnt += __popcll(m);
-        if (masks && part == 0) masks[oc] = m;
-    }
-    if (part == 0) counts[oc] = cnt;
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void status_store(unsigned long long *p, unsigned long long v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-__global__ void copy_last_kernel(const int32_t *v, int n, int32_t *out) { *out = n > 0 ? v[n - 1] : 0; }
+// Per-column counts and their inclusive scan (oz_ptr) in one launch.  16 lanes share an output column (one
+// input column (k0, k1) each, K0*K1 = 9 of them busy for a 3x3x3 kernel), so the fibers that reach a column
+// are walked side by side and small grids still fill the chip; a workgroup takes 64 columns.  Workgroups
+// number themselves by a ticket (so every predecessor of a workgroup is already running), publish the sum
+// of their counts, and look back over their predecessors' status words, 64 at a time, until they meet one
+// that already knows its inclusive prefix.  `masks` (O2 <= 64 only, else null) keeps each column's bin mask
+// for the fill kernel; `total` (may be null) receives the number of output rows.
+__global__ __launch_bounds__(kCountThreads) void outcoords_count_kernel(OutArgs a, int32_t *oz_ptr,
+                                                                        unsigned long long *masks, int *state,
+                                                                        int32_t *total)
+{
+    __shared__ int s_ticket, s_last;
+    __shared__ int s_cnt[kCountCols];
+    const int ncol = a.B * a.O.n0 * a.O.n1;
+    const int nblocks = count_blocks(ncol);
+    unsigned long long *status = (unsigned long long *)(state + 2);
+    const int tid = threadIdx.x;
+    if (tid == 0) {
+        s_ticket = atomicAdd(&state[0], 1);
+        s_last = 0;
+    }
+    __syncthreads();
+    const int t = s_ticket;
+    const int part = tid % kColLanes, cl = tid / kColLanes;
+    const int oc = t * kCountCols + cl;
+    int cnt = 0;
+    if (oc < ncol) { // whole 16-lane groups take this branch together
+        const int nchunk = (a.O.n2 + 63) >> 6;
+        const int b = oc / (a.O.n0 * a.O.n1);
+        const int rem = oc - b * (a.O.n0 * a.O.n1);
+        const int o0 = rem / a.O.n1, o1 = rem % a.O.n1;
+        for (int ch = 0; ch < nchunk; ch++) {
+            const unsigned long long m = or_reduce16(column_mask(a, b, o0, o1, ch, part, kColLanes));
+            cnt += __popcll(m);
+            if (masks && part == 0) masks[oc] = m;
+        }
+    }
+    if (part == 0) s_cnt[cl] = cnt;
+    __syncthreads();
+    if (tid < kWave) {
+        const int lane = tid;
+        int incl = s_cnt[lane];
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const int v = __shfl_up(incl, off, kWave);
+            if (lane >= off) incl += v;
+        }
+        const int agg = __shfl(incl, kWave - 1, kWave);
+        int excl = 0;
+        if (t > 0) {
+            if (lane == 0) status_store(&status[t], kScanAggregate | (unsigned)agg);
+            for (int base = t - 1;;) {
+                const int idx = base - lane; // lane 0 looks at the nearest predecessor
+                const unsigned long long w = idx >= 0 ? status_load(&status[idx]) : kScanInclusive; // before the first: 0
+                const unsigned long long flag = w >> 62;
+                const unsigned long long has_incl = __ballot(flag == 2), empty = __ballot(flag == 0);
+                const int fi = has_incl ? __ffsll((long long)has_incl) - 1 : kWave; // nearest inclusive prefix
+                const unsigned long long need = fi >= kWave - 1 ? ~0ull : (2ull << fi) - 1ull;
+                if (empty & need) { // a predecessor on the way has not published yet
+                    __builtin_amdgcn_s_sleep(1);
+                    continue;
+                }
+                int v = lane <= fi ? (int)(unsigned)w : 0;
+#pragma unroll
+                for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+                excl += v;
+                if (fi < kWave) break;
+                base -= kWave;
+            }
+        }
+        if (lane == 0) status_store(&status[t], kScanInclusive | (unsigned)(excl + agg));
+        const int c = t * kCountCols + lane;
+        if (c < ncol) oz_ptr[c] = excl + incl;
+        if (lane == 0) {
+            if (t == nblocks - 1 && total) *total = excl + agg;
+            // this workgroup reads no status word any more
+            if (atomicAdd(&state[1], 1) == nblocks - 1) s_last = 1;
+        }
+    }
+    __syncthreads();
+    if (s_last) { // every workgroup has finished its look-back: leave the state as it was found
+        for (int i = tid; i < nblocks; i += kCountThreads) status_store(&status[i], 0ull);
+        if (tid == 0) {
+            __hip_atomic_store(&state[0], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&state[1], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
 
 // oz_ptr holds the inclusive scan of the counts; one thread writes the bins of one column.
 __global__ __launch_bounds__(kThreads) void outcoords_fill_kernel(OutArgs a, const int32_t *oz_ptr, int32_t *oz_idx,
@@ -767,7 +847,7 @@ void sph_set_error(const char *fmt, ...)
 }
 
 SPH_EXPORT const char *sph_last_error(void) { return g_err; }
-SPH_EXPORT int sph_abi_version(void) { return 3; }
+SPH_EXPORT int sph_abi_version(void) { return 4; }
 SPH_EXPORT int sph_book_tiles(int rows) { return rows <= 0 ? 0 : sph_div_up(rows, R); }
 SPH_EXPORT int sph_book_cap(int KV) { return KV * (R / SPH_GROUP); }
 
@@ -867,23 +947,20 @@ SPH_EXPORT int sph_outcoords_blocks(const sph_geom *g)
     return sph_div_up(g->B * g->O[0] * g->O[1], kThreads);
 }
 
-static size_t outcoords_scan_bytes(long ncol)
+// int32 entries of the scratch the two calls share: the state of the scan across workgroups (two counters
+// and a 64-bit status word per workgroup of the count kernel) and, when a column's bins fit one 64-bit
+// mask, the masks behind it
+SPH_EXPORT int sph_outcoords_state_ints(const sph_geom *g)
 {
-    size_t bytes = 0;
-    hipError_t e = rocprim::inclusive_scan(nullptr, bytes, (int32_t *)nullptr, (int32_t *)nullptr, (size_t)(ncol > 0 ? ncol : 1),
-                                           rocprim::plus<int32_t>(), (hipStream_t)0);
-    return e == hipSuccess ? bytes + 8 : 0;
+    SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_state_ints: bad geometry");
+    return (int)scan_state_ints((long)g->B * g->O[0] * g->O[1]);
 }
 
-// int32 entries of the scratch the two calls share: the scan's temporary storage and, when a
-// column's bins fit one 64-bit mask, the masks (8-byte aligned behind it)
 SPH_EXPORT int sph_outcoords_scratch_ints(const sph_geom *g)
 {
     SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_scratch_ints: bad geometry");
     const long ncol = (long)g->B * g->O[0] * g->O[1];
-    const size_t scan = outcoords_scan_bytes(ncol);
-    SPH_REQUIRE(scan != 0, SPH_ERR_LAUNCH, "sph_outcoords_scratch_ints: temporary storage query failed");
-    const long n = (long)((scan + 7) / 8 * 2) + (g->O[2] <= 64 ? 2 * ncol : 0);
+    const long n = scan_state_ints(ncol) + (g->O[2] <= 64 ? 2 * ncol : 0);
     SPH_REQUIRE(n < 2147483647L, SPH_ERR_UNSUPPORTED, "sph_outcoords_scratch_ints: grid too large");
     return (int)n;
 }
@@ -891,8 +968,7 @@ SPH_EXPORT int sph_outcoords_scratch_ints(const sph_geom *g)
 static unsigned long long *outcoords_masks(const sph_geom *g, int32_t *scratch)
 {
     if (g->O[2] > 64) return nullptr;
-    const long ncol = (long)g->B * g->O[0] * g->O[1];
-    return (unsigned long long *)(scratch + (outcoords_scan_bytes(ncol) + 7) / 8 * 2);
+    return (unsigned long long *)(scratch + scan_state_ints((long)g->B * g->O[0] * g->O[1]));
 }
 
 static OutArgs out_args(const int32_t *z_idx, const int32_t *z_ptr, int in_rows, const sph_geom *g)
@@ -905,30 +981,23 @@ static OutArgs out_args(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
     return a;
 }
 
+static int outcoords_count(const char *who, const int32_t *z_idx, const int32_t *z_ptr, int in_rows, const sph_geom *g,
+                           int32_t *oz_ptr, int32_t *scratch, int32_t *total, void *stream)
+{
+    SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "%s: bad geometry", who);
+    SPH_REQUIRE(z_ptr && oz_ptr && scratch && in_rows >= 0 && (in_rows == 0 || z_idx), SPH_ERR_ARG, "%s: null argument", who);
+    SPH_REQUIRE((uintptr_t)scratch % 8 == 0, SPH_ERR_ARG, "%s: scratch must be 8-byte aligned", who);
+    const long ncol = (long)g->B * g->O[0] * g->O[1];
+    hipLaunchKernelGGL(outcoords_count_kernel, dim3(count_blocks(ncol)), dim3(kCountThreads), 0, (hipStream_t)stream,
+                       out_args(z_idx, z_ptr, in_rows, g), oz_ptr, outcoords_masks(g, scratch), (int *)scratch, total);
+    return sph_check_launch(who);
+}
+
 SPH_EXPORT int sph_outcoords_count(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
                                    const sph_geom *g, int32_t *oz_ptr, int32_t *scratch,
                                    int32_t *total_dev, void *stream)
 {
-    SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_count: bad geometry");
-    SPH_REQUIRE(z_ptr && oz_ptr && scratch && in_rows >= 0 && (in_rows == 0 || z_idx),
-                SPH_ERR_ARG, "sph_outcoords_count: null argument");
-    SPH_REQUIRE((uintptr_t)scratch % 8 == 0, SPH_ERR_ARG, "sph_outcoords_count: scratch must be 8-byte aligned");
-    hipStream_t st = (hipStream_t)stream;
-    const int ncol = g->B * g->O[0] * g->O[1];
-    hipLaunchKernelGGL(outcoords_count_kernel, dim3(sph_div_up(ncol, kColsPerBlock)), dim3(kThreads), 0, st,
-                       out_args(z_idx, z_ptr, in_rows, g), oz_ptr, outcoords_masks(g, scratch));
-    int rc = sph_check_launch("sph_outcoords_count");
-    if (rc) return rc;
-    size_t bytes = outcoords_scan_bytes(ncol);
-    SPH_REQUIRE(bytes != 0, SPH_ERR_LAUNCH, "sph_outcoords_count: temporary storage query failed");
-    hipError_t e = rocprim::inclusive_scan((void *)scratch, bytes, oz_ptr, oz_ptr, (size_t)ncol, rocprim::plus<int32_t>(), st);
-    if (e != hipSuccess) {
-        sph_set_error("sph_outcoords_count: scan: %s", hipGetErrorString(e));
-        return SPH_ERR_LAUNCH;
-    }
-    if (!total_dev) return SPH_OK; // the caller reads the last element of oz_ptr itself: one launch less
-    hipLaunchKernelGGL(copy_last_kernel, dim3(1), dim3(1), 0, st, (const int32_t *)oz_ptr, ncol, total_dev);
-    return sph_check_launch("sph_outcoords_count(total)");
+    return outcoords_count("sph_outcoords_count", z_idx, z_ptr, in_rows, g, oz_ptr, scratch, total_dev, stream);
 }
 
 SPH_EXPORT int sph_outcoords_fill(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,

@@ -206,24 +206,31 @@ class RuleBook:
     def build(cls, z_idx, z_ptr, batch, in_shape, out_shape, kernel, stride, padding,
               dilation=(1, 1, 1), weight=None):
         """Strided rules (replaces get_rules, rules.cu:405-486): output coordinates
-        (oz_ptr inclusive scan, oz_idx ascending per column) and pairs.  One
-        device->host read of the output row count, as in the reference (rules.cu:461)."""
+        (oz_ptr inclusive scan, oz_idx ascending per column) and pairs.  One wait for the
+        output row count, as in the reference (rules.cu:461): the count kernel writes it to pinned
+        host memory, so the wait is a stream synchronisation and no copy."""
         _check_index_tensors(z_idx, z_ptr, batch, in_shape)
         lib = L.lib()
         dev = z_ptr.device
         g = L.make_geom(batch, in_shape, out_shape, kernel, stride, padding, dilation)
         if min(int(v) for v in out_shape) <= 0:
             raise L.SphconvError("empty output grid %s" % (list(out_shape),))
-        nblk = lib.sph_outcoords_scratch_ints(C.byref(g))
-        if nblk < 0:
-            L.check(nblk)
+        nints = lib.sph_outcoords_scratch_ints(C.byref(g))
+        if nints < 0:
+            L.check(nints)
         oz_ptr = torch.empty((int(batch), int(out_shape[0]), int(out_shape[1])), dtype=torch.int32, device=dev)
-        scratch = torch.empty(nblk + (nblk & 1), dtype=torch.int32, device=dev)
+        scratch, total = _outcoords_workspace(dev, nints)
         n_in = int(z_idx.shape[0])
-        # no separate total: the inclusive scan's last element is read instead (one launch less)
-        L.check(lib.sph_outcoords_count(L.ptr(z_idx), L.ptr(z_ptr), n_in, C.byref(g), L.ptr(oz_ptr),
-                                        L.ptr(scratch), None, L.stream()))
-        out_rows = int(oz_ptr.view(-1)[-1].item())
+        stream = torch.cuda.current_stream(dev)
+        try:
+            # one launch: counts, their scan into oz_ptr, and the row count written straight to pinned host memory
+            L.check(lib.sph_outcoords_count(L.ptr(z_idx), L.ptr(z_ptr), n_in, C.byref(g), L.ptr(oz_ptr),
+                                            L.ptr(scratch), total.data_ptr(), stream.cuda_stream))
+            stream.synchronize()             # the one wait of a strided layer (the reference's is rules.cu:461)
+        except Exception:
+            _WORKSPACES.pop(_workspace_key(dev), None)   # the scan's state may not be zero any more
+            raise
+        out_rows = int(total[0])
         oz_idx = torch.empty(out_rows, dtype=torch.int32, device=dev)
         L.check(lib.sph_outcoords_fill(L.ptr(z_idx), L.ptr(z_ptr), n_in, C.byref(g), L.ptr(scratch),
                                        L.ptr(oz_ptr), L.ptr(oz_idx), out_rows, L.stream()))
@@ -328,6 +335,29 @@ class RuleBook:
     def tile_grid_shape(self, tile_size: Sequence[int] = (2, 2)) -> List[int]:
         """conv.py:32-38"""
         return [-(-self.out_shape[0] // int(tile_size[0])), -(-self.out_shape[1] // int(tile_size[1]))]
+
+
+# Scratch of the output-coordinate kernels, kept per (device, stream): the head of it is the state of the
+# scan across workgroups, which must be zero when a count is enqueued and is left zero by it, so it is
+# zeroed once, when it is allocated.  With it, one pinned host int that receives the output row count.
+_WORKSPACES = {}
+
+
+def _workspace_key(dev):
+    dev = torch.device(dev)
+    index = dev.index if dev.index is not None else torch.cuda.current_device()
+    return (index, torch.cuda.current_stream(index).cuda_stream)
+
+
+def _outcoords_workspace(dev, nints: int):
+    key = _workspace_key(dev)
+    ws = _WORKSPACES.get(key)
+    if ws is None or ws[0].numel() < nints:
+        scratch = torch.zeros(max(nints + (nints & 1), 1 << 16), dtype=torch.int32, device=dev)
+        total = ws[1] if ws is not None else torch.zeros(1, dtype=torch.int32).pin_memory()
+        ws = (scratch, total)
+        _WORKSPACES[key] = ws
+    return ws
 
 
 def _check_index_tensors(z_idx, z_ptr, batch, shape):

@@ -259,8 +259,9 @@ def test_unsorted_long_fibers_take_the_general_join():
 
 
 def test_outcoords_total_is_optional():
-    """sph_outcoords_count writes the output row count to *total_dev when given one and skips that launch
-    when not; either way the count is the last element of the scanned oz_ptr."""
+    """sph_outcoords_count writes the output row count to *total_dev when given one; either way the count is
+    the last element of the scanned oz_ptr.  The head of the scratch (the state of the scan across workgroups)
+    must be zero on entry and is zero again afterwards, so one zeroed scratch serves call after call."""
     import ctypes as C
     from sphconv_amd import _lib as L
     rng = np.random.default_rng(5)
@@ -271,16 +272,50 @@ def test_outcoords_total_is_optional():
     lib = L.lib()
     g = L.make_geom(B, shape, out_shape, [3, 3, 3], [2, 2, 2], [1, 1, 1], [1, 1, 1])
     n = lib.sph_outcoords_scratch_ints(C.byref(g))
+    ns = lib.sph_outcoords_state_ints(C.byref(g))
+    assert 0 < ns <= n
     ptrs = []
+    scratch = torch.zeros(n + (n & 1), dtype=torch.int32, device="cuda:0")
     for with_total in (True, False):
         oz_ptr = torch.empty((B, out_shape[0], out_shape[1]), dtype=torch.int32, device="cuda:0")
-        scratch = torch.empty(n + (n & 1), dtype=torch.int32, device="cuda:0")
         total = torch.full((1,), -7, dtype=torch.int32, device="cuda:0")
         L.check(lib.sph_outcoords_count(L.ptr(zi), L.ptr(zp), int(zi.shape[0]), C.byref(g), L.ptr(oz_ptr),
                                         L.ptr(scratch), L.ptr(total) if with_total else None, L.stream()))
         torch.cuda.synchronize()
         assert int(total.item()) == (int(oz_ptr.view(-1)[-1].item()) if with_total else -7)
+        assert int(scratch[:ns].abs().sum().item()) == 0
         ptrs.append(oz_ptr.cpu().numpy())
     assert np.array_equal(ptrs[0], ptrs[1])
     book = RuleBook.build(zi, zp, B, shape, out_shape, [3, 3, 3], [2, 2, 2], [1, 1, 1])
     assert np.array_equal(book.oz_ptr.cpu().numpy(), ptrs[0]) and book.out_rows == int(ptrs[0].reshape(-1)[-1])
+
+
+@pytest.mark.parametrize("shape,p", [([40, 700, 20], 0.02), ([64, 1024, 70], 0.05), ([3, 21, 9], 0.5)])
+def test_outcoords_scan_over_many_workgroups(shape, p):
+    """The scan of the per-column counts runs inside the count kernel, across its workgroups of 64 columns:
+    grids of one workgroup, of hundreds (look-back over several windows of 64 predecessors) and with more
+    than 64 bins (no masks kept), twice in a row on the same scratch, against numpy's cumsum."""
+    import ctypes as C
+    from sphconv_amd import _lib as L
+    rng = np.random.default_rng(shape[1])
+    B = 3
+    idx = np.argwhere(rng.random((B, *shape)) < p).astype(np.int32)
+    _, z_idx, z_ptr, _ = H.csr_from_indices(idx, B, shape)
+    out_shape = H.out_shape_of(shape, [3, 3, 3], [2, 2, 2], [1, 1, 1])
+    occ = np.zeros((B, *shape), np.float32)
+    occ[tuple(idx.T)] = 1
+    act = torch.nn.functional.conv3d(torch.tensor(occ)[:, None], torch.ones((1, 1, 3, 3, 3)), stride=2, padding=1)[:, 0] != 0
+    want = np.cumsum(act.sum(3).numpy().reshape(-1)).astype(np.int32)
+    lib = L.lib()
+    g = L.make_geom(B, shape, out_shape, [3, 3, 3], [2, 2, 2], [1, 1, 1], [1, 1, 1])
+    n = lib.sph_outcoords_scratch_ints(C.byref(g))
+    scratch = torch.zeros(n + (n & 1), dtype=torch.int32, device="cuda:0")
+    zi, zp = G.t(z_idx), G.t(z_ptr)
+    for _ in range(2):
+        oz_ptr = torch.full((B, out_shape[0], out_shape[1]), -1, dtype=torch.int32, device="cuda:0")
+        total = torch.zeros(1, dtype=torch.int32).pin_memory()
+        L.check(lib.sph_outcoords_count(L.ptr(zi), L.ptr(zp), int(zi.shape[0]), C.byref(g), L.ptr(oz_ptr),
+                                        L.ptr(scratch), total.data_ptr(), L.stream()))
+        torch.cuda.current_stream().synchronize()
+        assert int(total[0]) == int(want[-1])            # written by the kernel to pinned host memory
+        assert np.array_equal(oz_ptr.cpu().numpy().reshape(-1), want)
