@@ -154,6 +154,21 @@ int sph_outcoords_fill(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
                        const sph_geom *g, const int32_t *scratch, int32_t *oz_ptr,
                        int32_t *oz_idx, int out_rows, void *stream);
 
+/* sph_outcoords_count for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * kernels and results as sph_outcoords_count, but the scratch is an array of the library's own
+ * (8.1 MiB of static device memory on each GPU the library runs on, held until the process ends),
+ * so the call allocates and frees nothing.  It serves grids of up to SPH_STATIC_MAX_COLUMNS output
+ * columns (B * O[0] * O[1]) and refuses larger ones with SPH_ERR_UNSUPPORTED.  *scratch_out (may be
+ * null) receives the array's device address on the current GPU: pass it as `scratch` to
+ * sph_outcoords_fill.  Every call on a GPU shares that GPU's array, which keeps the last call's
+ * contents (the call clears the part that must start at zero): calls that overlap on one GPU race,
+ * and a second call overwrites the bin masks a pending sph_outcoords_fill of the first would read. */
+#define SPH_STATIC_MAX_COLUMNS 1048576
+int sph_outcoords_count_static(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
+                               const sph_geom *g, int32_t *oz_ptr, int32_t *total_dev,
+                               const int32_t **scratch_out, void *stream);
+
 /* Conversions between the rule book and the reference's padded tensors
  * `rules [NTile,KV,2,tile_n_max]`, `rule_size [NTile,KV]` (rules.cu:364-369).
  * nbr is scratch of out_rows*KV int32 (forward) / in_rows*KV (transposed). */

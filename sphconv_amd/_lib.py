@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libsphconv_hip.so")
 
 TILE_ROWS = 128
 GROUP = 16
+STATIC_MAX_COLUMNS = 1 << 20     # SPH_STATIC_MAX_COLUMNS of the header
 
 F32, F16, BF16, I8 = 0, 1, 2, 3
 _DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.int8: I8}
@@ -58,6 +59,7 @@ _SIGNATURES = {
     "sph_outcoords_scratch_ints": (_I, [C.POINTER(Geom)]),
     "sph_outcoords_state_ints": (_I, [C.POINTER(Geom)]),
     "sph_outcoords_count": (_I, [_P, _P, _I, C.POINTER(Geom), _P, _P, _P, _P]),
+    "sph_outcoords_count_static": (_I, [_P, _P, _I, C.POINTER(Geom), _P, _P, C.POINTER(C.c_void_p), _P]),
     "sph_outcoords_fill": (_I, [_P, _P, _I, C.POINTER(Geom), _P, _P, _P, _I, _P]),
     "sph_rules_to_padded_count": (_I, [C.POINTER(Book), _P, C.POINTER(Geom), _I, _I, _P, _P, _P]),
     "sph_rules_to_padded_fill": (_I, [_P, C.POINTER(Geom), _I, _I, _P, _I, _I, _I, _P, _P]),

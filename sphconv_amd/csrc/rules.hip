@@ -9,6 +9,7 @@
 #include "pack.h"
 
 #include <cstring>
+#include <mutex>
 
 namespace {
 
@@ -998,6 +999,63 @@ SPH_EXPORT int sph_outcoords_count(const int32_t *z_idx, const int32_t *z_ptr, i
                                    int32_t *total_dev, void *stream)
 {
     return outcoords_count("sph_outcoords_count", z_idx, z_ptr, in_rows, g, oz_ptr, scratch, total_dev, stream);
+}
+
+// ---------------------------------------------------------------------------
+// sph_outcoords_count for callers that cannot allocate: the scratch is an array of the library's own.
+// Each GPU holds its own copy of the array at its own address, found once per device.
+// ---------------------------------------------------------------------------
+constexpr long kStaticCols = SPH_STATIC_MAX_COLUMNS; // output columns (B * O0 * O1) the library's own scratch provides for
+constexpr long kStaticInts = 2 + 2 * ((kStaticCols + kCountCols - 1) / kCountCols) + 2 * kStaticCols;
+static __device__ __align__(256) int32_t sph_static_scratch[kStaticInts]; // 8.1 MiB per GPU
+constexpr int kMaxDevices = 64;
+static int32_t *g_static_ptr[kMaxDevices];
+static std::mutex g_static_mutex;
+
+// device address of this GPU's copy of the array (the array's name is no device address in host code)
+static int static_scratch_ptr(const char *who, int32_t **out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        sph_set_error("%s: hipGetDevice: %s (device %d)", who, hipGetErrorString(e), dev);
+        return SPH_ERR_LAUNCH;
+    }
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (!g_static_ptr[dev]) {
+        int32_t *p = nullptr;
+        e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(sph_static_scratch));
+        if (e != hipSuccess || !p) {
+            sph_set_error("%s: hipGetSymbolAddress: %s", who, hipGetErrorString(e));
+            return SPH_ERR_LAUNCH;
+        }
+        g_static_ptr[dev] = p;
+    }
+    *out = g_static_ptr[dev];
+    return SPH_OK;
+}
+
+SPH_EXPORT int sph_outcoords_count_static(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
+                                          const sph_geom *g, int32_t *oz_ptr, int32_t *total_dev,
+                                          const int32_t **scratch_out, void *stream)
+{
+    const char *who = "sph_outcoords_count_static";
+    SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "%s: bad geometry", who);
+    const long ncol = (long)g->B * g->O[0] * g->O[1];
+    SPH_REQUIRE(ncol <= kStaticCols, SPH_ERR_UNSUPPORTED,
+                "%s: %ld output columns (B*O0*O1), the library's own scratch provides for %ld: use sph_outcoords_count "
+                "with a scratch of the caller's", who, ncol, kStaticCols);
+    int32_t *ptr = nullptr;
+    int rc = static_scratch_ptr(who, &ptr);
+    if (rc) return rc;
+    // the scan's state must start at zero; a launch leaves it so, but one that was cut short would not
+    const long n = scan_state_ints(ncol);
+    hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, ptr, n, 0);
+    rc = sph_check_launch(who);
+    if (rc) return rc;
+    rc = outcoords_count(who, z_idx, z_ptr, in_rows, g, oz_ptr, ptr, total_dev, stream);
+    if (rc == SPH_OK && scratch_out) *scratch_out = ptr;
+    return rc;
 }
 
 SPH_EXPORT int sph_outcoords_fill(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
