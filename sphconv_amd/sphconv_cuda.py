@@ -14,6 +14,7 @@ unchanged with ``sphconv_amd.sphconv_cuda``.  Differences, all additive:
 * bad arguments raise ``SphconvError`` / ``ValueError`` instead of aborting.
 """
 import ctypes as C
+import weakref
 from typing import List, Optional, Sequence
 
 import torch
@@ -23,14 +24,29 @@ from .rulebook import RuleBook
 
 __version__ = "hip-gfx950"
 
+# Packed copies of weights seen while no gradient is being recorded (inference): one per (weight storage,
+# form), valid as long as the tensor object lives and its version counter, which every in-place update
+# bumps, has not moved.
+_PACKED_CACHE = {}
+
+
 def _packed_weight(weight: torch.Tensor, transpose: bool, reverse: bool = False) -> torch.Tensor:
     """weight [KV, a, b] -> fragment-ordered copy for the contraction over ``a``
     (``transpose``: over ``b``, i.e. with W[k]^T; ``reverse``: offsets in reverse order, W[KV-1-k]).
-    Packed on every call: the weight may have been updated in place since the last one."""
-    lib = L.lib()
+    While gradients are being recorded the copy is made on every call (an optimiser step may follow);
+    under ``torch.no_grad()`` it is kept with the weight and reused until the weight changes."""
     w = weight.detach()
     if not w.is_contiguous():
         w = w.contiguous()
+    cache_key = None
+    if not torch.is_grad_enabled() and w.data_ptr() == weight.data_ptr():
+        base = weight._base if weight._base is not None else weight
+        cache_key = (id(base), bool(transpose), bool(reverse))
+        state = (base._version, w.data_ptr(), tuple(w.shape), w.dtype)
+        hit = _PACKED_CACHE.get(cache_key)
+        if hit is not None and hit[0]() is base and hit[1] == state:
+            return hit[2]
+    lib = L.lib()
     kv, a, b = w.shape
     kdim, ndim = (b, a) if transpose else (a, b)
     skk, sn = (1, b) if transpose else (b, 1)
@@ -43,6 +59,8 @@ def _packed_weight(weight: torch.Tensor, transpose: bool, reverse: bool = False)
     if reverse:                                  # start at the last offset and walk backwards
         first, sk = first + (kv - 1) * a * b * w.element_size(), -a * b
     L.check(lib.sph_weight_pack(dt, first, kv, kdim, ndim, sk, skk, sn, L.ptr(packed), L.stream()))
+    if cache_key is not None:
+        _PACKED_CACHE[cache_key] = (weakref.ref(base, lambda _r, k=cache_key: _PACKED_CACHE.pop(k, None)), state, packed)
     return packed
 
 

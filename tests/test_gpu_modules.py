@@ -275,3 +275,26 @@ def test_config4_encoder_full_size_layer_by_layer():
             assert 0.2 < (want > 0).mean() < 0.9 and 1e-2 < np.abs(want).mean() < 1e2, (i, np.abs(want).mean())
             x = y
     assert [x.D, x.W, x.H] == [4, 128, 4] and x.feature.shape[1] == 64
+
+
+def test_packed_weight_is_kept_under_no_grad_and_follows_updates():
+    """Under torch.no_grad() the fragment-ordered copy of a weight is made once and reused until the weight's
+    version counter moves (an in-place update); while gradients are recorded it is made on every call."""
+    from sphconv_amd import sphconv_cuda as ext
+    B, shape = 1, [8, 16, 8]
+    idx, feat = _inputs(3, B, shape, 16)
+    conv = sphconv.SubMConv3d(16, 32, 3).to(G.DEV).half()
+    x = sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx))
+    w = conv.weight.view(-1, 16, 32)
+    with torch.no_grad():
+        p1 = ext._packed_weight(w, False)
+        assert ext._packed_weight(conv.weight.view(-1, 16, 32), False) is p1        # another view of the same parameter
+        assert ext._packed_weight(w, True) is not p1                                  # other form, other copy
+        y1 = conv(x).feature.clone()
+        conv.weight.mul_(2.0)                                                         # bumps the version counter
+        p2 = ext._packed_weight(w, False)
+        assert p2 is not p1 and not torch.equal(p2, p1)
+        y2 = conv(x).feature
+    torch.testing.assert_close(y2.float(), 2 * y1.float(), rtol=2e-3, atol=2e-3)
+    with torch.enable_grad():
+        assert ext._packed_weight(w, False) is not ext._packed_weight(w, False)
