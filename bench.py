@@ -11,11 +11,15 @@ the scan's index arrays, features and weights already resident in HBM.
 The timed steps are dealt to a few HIP streams (--streams, default 3): every step redoes all
 of its work into per-stream buffers, but the rule kernel of one scan can run beside the
 convolution of another.  `one_stream_ms_per_step` is the same step with one scan at a time.
+The steps walk through --scans resident copies of the scan (more memory than the last-level
+cache holds); the timed loop of --steps steps is repeated --repeats times and the median counts,
+after the per-kernel section has settled the device.
 
 Prints ONE JSON line:  value = active voxels / second over the timed steps,
 plus `rulegen_ms_per_scan`, a `roofline` object for the dominant kernel (live
-HIP-event timing of that kernel alone) and a `cpu_baseline` object (the CPU
-restatement of the reference algorithm under oracle/, timed on this host).
+HIP-event timing of that kernel alone), an `at_120k` object (the same step on a scan of the
+size BASELINE's metric names) and a `cpu_baseline` object (the CPU restatement of the reference
+algorithm under oracle/, timed on this host).
 """
 import argparse
 import json
@@ -27,11 +31,6 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the two candidates for "dominant kernel" at the default workload
-# (seed 0), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script scaled by a
-# 256 MiB copy (factors 2.000 / 1.000); commands and raw values: profiles/bench_headline_subm64_f16.md.
-# None for any other workload.
-MEASURED_TRAFFIC_BYTES = {"conv": 9595 * 1024 * 2 + 11924 * 1024, "rules": 1067 * 1024 * 2 + 3461 * 1024}
 
 
 def parse():
@@ -41,6 +40,14 @@ def parse():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--streams", type=int, default=3, help="HIP streams the timed scans are dealt to")
+    ap.add_argument("--scans", type=int, default=24,
+                    help="resident copies of the scan the timed steps walk through (24 x 13 MB is more than the "
+                         "256 MB last-level cache holds)")
+    ap.add_argument("--repeats", type=int, default=7, help="the timed loop of `steps` steps is repeated this often; "
+                                                           "the median is reported")
+    ap.add_argument("--voxels", type=int, default=120000,
+                    help="also measure the same step on a scan of about this many voxels (the generator's column "
+                         "occupancy raised), reported as 'at_120k'; 0: skip")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--backward", action="store_true",
                     help="also time dgrad (transposed rule book + kernel) and wgrad of the same layer; "
@@ -267,6 +274,159 @@ def configs_ms(torch, seed, iters):
     return out
 
 
+def kernel_sources_digest():
+    """sha256 over the sources of the two kernels whose HBM traffic is on record (what a counter run was
+    taken on): the recorded traffic is only reported while these files are what it was measured on."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in ("conv.hip", "rules.hip", "common.h", "pack.h"):
+        with open(os.path.join(ROOT, "sphconv_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def recorded_traffic(kernel_key, voxels, seed):
+    """HBM bytes per launch of a kernel from profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+    scaled by a copy of known size), or None when the record is for other sources, another seed or another
+    scan size."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None
+    if rec.get("sources_sha256") != kernel_sources_digest() or rec.get("seed") != seed:
+        return None
+    for e in rec.get("kernels", []):
+        if e.get("key") == kernel_key and e.get("voxels") == voxels:
+            return e.get("hbm_bytes")
+    return None
+
+
+class Workload:
+    """One scan size of the benchmark: `copies` device-resident copies of the scan (index arrays and
+    features in separate allocations, so that the timed steps walk through more memory than the 256 MB
+    last-level cache holds), and the timings of the step on it."""
+
+    def __init__(self, torch, d, ic, oc, w, copies, seed):
+        self.torch = torch
+        self.d, self.ic, self.oc, self.w = d, ic, oc, w
+        self.shape, self.B = d["spatial_shape"], d["batch"]
+        self.n = int(d["z_idx"].shape[0])
+        dev = w.device
+        gen = torch.Generator(device=dev).manual_seed(seed)
+        zi, zp = torch.tensor(d["z_idx"]), torch.tensor(d["z_ptr"])
+        self.scans = []
+        for _ in range(copies):
+            feat = torch.randn((self.n, ic), device=dev, generator=gen).half()
+            self.scans.append((feat, zi.to(dev).clone(), zp.to(dev).clone()))
+        self.footprint = copies * (self.n * ic * 2 + self.n * 4 + zp.numel() * 4)
+
+    def step(self, i):
+        """rule generation (the weight is put in MFMA fragment order by extra workgroups of the same launch,
+        every step) + forward, on copy i of the scan."""
+        from sphconv_amd import sphconv_cuda as ext
+        from sphconv_amd.rulebook import RuleBook
+        feat, z_idx, z_ptr = self.scans[i % len(self.scans)]
+        book, packed = RuleBook.build_subm(z_idx, z_ptr, self.B, self.shape, [3, 3, 3], weight=self.w)
+        return book, ext.rule_conv(feat, self.w, book, None, self.n, packed=packed)
+
+    def time_one_stream(self, steps, warmup, repeats):
+        torch = self.torch
+        for i in range(warmup):
+            self.step(i)
+        torch.cuda.synchronize()
+        times = []
+        for r in range(repeats):
+            t0 = time.perf_counter()
+            for i in range(steps):
+                self.step(r * steps + i)
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) / steps * 1e3)
+        return sorted(times)[len(times) // 2], times
+
+    def time_pipelined(self, steps, warmup, repeats, streams):
+        """The same two launches per scan, scans dealt to a few HIP streams so that the rule kernel of one scan
+        runs beside the convolution of another (a 100k-voxel scan fills neither kernel's grid); buffers are
+        allocated once per stream slot, every step redoes all the work."""
+        torch = self.torch
+        from sphconv_amd.pipeline import ScanPipeline
+        pipe = ScanPipeline(self.w, self.B, self.shape, max_voxels=self.n, streams=streams)
+        for i in range(warmup):
+            pipe.submit(*self.scans[i % len(self.scans)], wait_inputs=False)
+        pipe.synchronize()
+        torch.cuda.synchronize()
+        times = []
+        last = None
+        for r in range(repeats):
+            t0 = time.perf_counter()
+            for i in range(steps):
+                k = (r * steps + i) % len(self.scans)
+                last = (pipe.submit(*self.scans[k], wait_inputs=False), k)   # inputs are resident and complete
+            pipe.synchronize()
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) / steps * 1e3)
+        (out_p, _slot), k = last
+        _, out = self.step(k)
+        assert torch.equal(out_p, out)
+        return sorted(times)[len(times) // 2], times
+
+    def time_kernels(self, iters, backward=False, rng=None):
+        """Each kernel alone: HIP events on the launch stream around `iters` back-to-back launches."""
+        import ctypes as C
+        from sphconv_amd import _lib as L
+        from sphconv_amd import sphconv_cuda as ext
+        torch = self.torch
+        lib = L.lib()
+        feat, z_idx, z_ptr = self.scans[0]
+        n, ic, oc, w = self.n, self.ic, self.oc, self.w
+        book, out = self.step(0)
+        self.pairs = book.num_pairs()
+        g = book.geom()
+        bk = book.fwd.struct()
+        stream = L.stream()
+        res = {}
+        res["rulegen_ms"] = event_ms(lambda: lib.sph_rules_build(z_idx.data_ptr(), z_ptr.data_ptr(), n, z_idx.data_ptr(),
+                                                                 z_ptr.data_ptr(), n, C.byref(g), 0, C.byref(bk), stream),
+                                     iters, torch)
+        packed = ext._packed_weight(w, False)
+        out_buf = torch.empty((n, oc), dtype=torch.float16, device=w.device)
+        epi = L.Epilogue(None, None, 0)
+        res["conv_forward_ms"] = event_ms(lambda: lib.sph_conv_apply(L.F16, feat.data_ptr(), n, ic, packed.data_ptr(), oc,
+                                                                     C.byref(bk), C.byref(epi), out_buf.data_ptr(), stream),
+                                          iters, torch)
+        res["weight_pack_ms"] = event_ms(lambda: lib.sph_weight_pack(L.F16, w.data_ptr(), 27, ic, oc, ic * oc, oc, 1,
+                                                                     packed.data_ptr(), stream), iters, torch)
+        assert torch.equal(out_buf, out)
+        if backward:
+            d_out = torch.randn((n, oc), device=w.device).half()
+            w_t = w.permute(0, 2, 1).contiguous()
+            res["transposed_rulegen_ms"] = event_ms(lambda: book._build(True), iters, torch)
+            book.transposed()
+            res["dgrad_ms"] = event_ms(lambda: ext.rule_conv_d_feature(d_out, w_t, book, None, None, n), iters, torch)
+            res["wgrad_ms"] = event_ms(lambda: ext.rule_conv_d_weight(feat, d_out, book, None), iters, torch)
+        e, P = 2, self.pairs
+        nt = book.fwd.ntiles
+        self.conv_bytes = n * ic * e + n * oc * e + 27 * ic * oc * e + 8 * P
+        self.rule_bytes = 4 * z_ptr.numel() + 4 * n + 8 * P + nt * (4 + 2 * 28)
+        res["rulegen_GBps"] = self.rule_bytes / (res["rulegen_ms"] * 1e-3) / 1e9
+        res["conv_GBps"] = self.conv_bytes / (res["conv_forward_ms"] * 1e-3) / 1e9
+        res["conv_TFLOPs"] = 2.0 * P * ic * oc / (res["conv_forward_ms"] * 1e-3) / 1e12
+        return res
+
+    def roofline(self, kern, seed):
+        """For the kernel that lasts longest: algorithmic bytes per launch / its average duration, against the
+        HBM peak."""
+        if kern["conv_forward_ms"] >= kern["rulegen_ms"]:
+            dom = ("conv_wave_kernel<f16,2,4,false>", self.conv_bytes, kern["conv_forward_ms"], "conv")
+        else:
+            dom = ("build_book_kernel<false>", self.rule_bytes, kern["rulegen_ms"], "rules")
+        achieved = dom[1] / (dom[2] * 1e-3) / 1e9
+        return {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic(dom[3], self.n, seed),
+                "kernel": dom[0], "algorithmic_bytes": dom[1], "kernel_ms": dom[2]}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -276,24 +436,16 @@ def main():
     import numpy as np
     import torch
 
-    from sphconv_amd import sphconv_cuda as ext
-    from sphconv_amd.pipeline import ScanPipeline
-    from sphconv_amd.rulebook import RuleBook
-    from sphconv_amd.synth import make_config
+    from sphconv_amd.synth import config2_with_voxels, make_config
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
     torch.cuda.set_device(0)
     ic = oc = 64
-    d = make_config(2, seed=args.seed)
-    shape, B = d["spatial_shape"], d["batch"]
-    n = int(d["z_idx"].shape[0])
     rng = np.random.default_rng(args.seed)
-    z_idx = torch.tensor(d["z_idx"], device=dev)
-    z_ptr = torch.tensor(d["z_ptr"], device=dev)
-    feat = torch.tensor(rng.standard_normal((n, ic)), dtype=torch.float32, device=dev).half()
     w = torch.tensor(rng.standard_normal((27, ic, oc)) * np.sqrt(2.0 / (27 * ic)), dtype=torch.float32,
                      device=dev).half()
+    d = make_config(2, seed=args.seed)
 
     if args.copy_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -303,100 +455,45 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    def step():
-        # rule generation (the weight is put in MFMA fragment order by extra workgroups of the
-        # same launch, every step) + forward
-        book, packed = RuleBook.build_subm(z_idx, z_ptr, B, shape, [3, 3, 3], weight=w)
-        return book, ext.rule_conv(feat, w, book, None, n, packed=packed)
+    def measure(d):
+        wl = Workload(torch, d, ic, oc, w, args.scans, args.seed)
+        # the per-kernel section goes first: its hundreds of launches settle clocks and caches, so that a short
+        # timed run (--steps 20) reads the same as a long one
+        iters = max(100, min(args.steps, 200))
+        kern = wl.time_kernels(iters, backward=args.backward, rng=rng)
+        one_ms, one_all = wl.time_one_stream(args.steps, max(args.warmup, 20), args.repeats)
+        ms, ms_all = wl.time_pipelined(args.steps, max(args.warmup, 20), args.repeats, args.streams)
+        return wl, kern, one_ms, ms, {"one_stream_ms": one_all, "pipelined_ms": ms_all}
 
-    # one scan at a time on one stream (latency of a scan)
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        book, out = step()
-    torch.cuda.synchronize()
-    one_stream_ms = (time.perf_counter() - t0) / args.steps * 1e3
-
-    # the timed steps: the same two launches per scan, scans dealt to a few HIP streams so that the
-    # rule kernel of one scan runs beside the convolution of another (a 95k-voxel scan fills neither
-    # kernel's grid); buffers are allocated once per stream slot, every step redoes all the work
-    pipe = ScanPipeline(w, B, shape, max_voxels=n, streams=args.streams)
-    for _ in range(args.warmup):
-        pipe.submit(feat, z_idx, z_ptr, wait_inputs=False)
-    pipe.synchronize()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        out_p, slot = pipe.submit(feat, z_idx, z_ptr, wait_inputs=False)   # inputs are resident and complete
-    pipe.synchronize()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
-    assert torch.equal(out_p, out)
-
-    # ---- per-kernel timings (HIP events on the launch stream) ------------------
-    P = book.num_pairs()
-    iters = max(20, min(args.steps, 200))
-    import ctypes as C
-    from sphconv_amd import _lib as L
-    lib = L.lib()
-    g = book.geom()
-    bk = book.fwd.struct()          # re-fills the buffers of the last step's book
-    stream = L.stream()
-    rulegen_ms = event_ms(lambda: lib.sph_rules_build(z_idx.data_ptr(), z_ptr.data_ptr(), n, z_idx.data_ptr(),
-                                                      z_ptr.data_ptr(), n, C.byref(g), 0, C.byref(bk), stream),
-                          iters, torch)
-    packed = ext._packed_weight(w, False)
-    out_buf = torch.empty((n, oc), dtype=torch.float16, device=dev)
-    epi = L.Epilogue(None, None, 0)
-    conv_ms = event_ms(lambda: lib.sph_conv_apply(L.F16, feat.data_ptr(), n, ic, packed.data_ptr(), oc,
-                                                  C.byref(bk), C.byref(epi), out_buf.data_ptr(), stream),
-                       iters, torch)
-    pack_ms = event_ms(lambda: lib.sph_weight_pack(L.F16, w.data_ptr(), 27, ic, oc, ic * oc, oc, 1,
-                                                   packed.data_ptr(), stream), iters, torch)
-    assert torch.equal(out_buf, out)
-    extra = {}
-    if args.backward:
-        d_out = torch.tensor(rng.standard_normal((n, oc)), dtype=torch.float32, device=dev).half()
-        w_t = w.permute(0, 2, 1).contiguous()
-        extra["transposed_rulegen_ms"] = event_ms(lambda: book._build(True), iters, torch)
-        book.transposed()
-        extra["dgrad_ms"] = event_ms(lambda: ext.rule_conv_d_feature(d_out, w_t, book, None, None, n), iters, torch)
-        extra["wgrad_ms"] = event_ms(lambda: ext.rule_conv_d_weight(feat, d_out, book, None), iters, torch)
-    e = 2
-    nt = book.fwd.ntiles
-    conv_bytes = n * ic * e + n * oc * e + 27 * ic * oc * e + 8 * P
-    rule_bytes = 4 * z_ptr.numel() + 4 * n + 8 * P + nt * (4 + 2 * 28)
-    conv_flops = 2.0 * P * ic * oc
-    if conv_ms >= rulegen_ms:
-        dom = {"kernel": "conv_wave_kernel<f16,2,4,false>", "bytes": conv_bytes, "ms": conv_ms, "key": "conv"}
-    else:
-        dom = {"kernel": "build_book_kernel<false>", "bytes": rule_bytes, "ms": rulegen_ms, "key": "rules"}
-    achieved = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBS,
-                "traffic": MEASURED_TRAFFIC_BYTES[dom["key"]] if args.seed == 0 else None, "kernel": dom["kernel"],
-                "algorithmic_bytes": dom["bytes"], "kernel_ms": dom["ms"]}
-
+    wl, kern, one_stream_ms, ms_per_step, repeats = measure(d)
+    n, P = wl.n, wl.pairs
     result = {
         "metric": "active voxels/sec, 3x3x3 subm conv 64->64 fp16 (rulegen + forward); rulegen ms/scan",
         "value": n / (ms_per_step * 1e-3), "unit": "voxels/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "config-2 generator (G2, seed %d): grid 64x2048x64, batch 1, %d active voxels, "
-                               "%d pairs; subm 3x3x3 64->64, fp16 storage / fp32 accumulate; scans dealt to %d HIP streams"
-                               % (args.seed, n, P, args.streams),
-                   "grid": shape, "batch": B, "voxels": n, "pairs": P, "channels": [ic, oc]},
-        "rulegen_ms_per_scan": rulegen_ms,
+                               "%d pairs; subm 3x3x3 64->64, fp16 storage / fp32 accumulate; the timed steps walk "
+                               "through %d resident copies of the scan (%d MB) on %d HIP streams; ms_per_step is the "
+                               "median of %d repeats of `steps` steps"
+                               % (args.seed, n, P, args.scans, wl.footprint >> 20, args.streams, args.repeats),
+                   "grid": wl.shape, "batch": wl.B, "voxels": n, "pairs": P, "channels": [ic, oc]},
+        "rulegen_ms_per_scan": kern["rulegen_ms"],
         "streams": args.streams, "one_stream_ms_per_step": one_stream_ms,
-        "kernels": {"rulegen_ms": rulegen_ms, "weight_pack_ms": pack_ms, "conv_forward_ms": conv_ms,
-                    "rulegen_GBps": rule_bytes / (rulegen_ms * 1e-3) / 1e9,
-                    "conv_GBps": conv_bytes / (conv_ms * 1e-3) / 1e9,
-                    "conv_TFLOPs": conv_flops / (conv_ms * 1e-3) / 1e12, **extra},
-        "roofline": roofline,
+        "one_stream_value": n / (one_stream_ms * 1e-3),
+        "repeats": repeats,
+        "kernels": kern,
+        "roofline": wl.roofline(kern, args.seed),
     }
+    if args.voxels > 0:
+        # the size BASELINE's metric names: the same generator with its column occupancy raised
+        d2, p2 = config2_with_voxels(args.voxels, seed=args.seed)
+        wl2, kern2, one2, ms2, rep2 = measure(d2)
+        result["at_120k"] = {
+            "workload": "config-2 generator with column occupancy %.3f: %d active voxels, %d pairs" % (p2, wl2.n, wl2.pairs),
+            "voxels": wl2.n, "pairs": wl2.pairs, "value": wl2.n / (ms2 * 1e-3), "unit": "voxels/s",
+            "ms_per_step": ms2, "one_stream_ms_per_step": one2, "rulegen_ms_per_scan": kern2["rulegen_ms"],
+            "kernels": kern2, "roofline": wl2.roofline(kern2, args.seed), "repeats": rep2}
     if args.callers:
         result["callers"] = callers_ms(torch, d, args.seed, 50)
     if args.configs:

@@ -71,10 +71,11 @@ def occupancy_g2(B: int, S0: int, S1: int, S2: int, p: float = 0.5, seed: int = 
     return occ
 
 
-def make_config(cfg: int, seed: int = 0, batch: int = None):
+def make_config(cfg: int, seed: int = 0, batch: int = None, p: float = None):
     """Occupancy of benchmark configuration ``cfg`` (1..5) -> dict with
     ``indices`` [N,4] (b,s0,s1,s2) int32, ``z_idx``, ``z_ptr`` and
-    ``spatial_shape`` = [S0,S1,S2], ``batch``."""
+    ``spatial_shape`` = [S0,S1,S2], ``batch``.  ``p`` overrides the generator's column occupancy
+    (0.6 for G1, 0.5 for G2), e.g. to reach a given number of voxels."""
     if cfg == 1:
         B, shape, gen = 1, (64, 512, 32), occupancy_g1
     elif cfg == 2:
@@ -87,10 +88,24 @@ def make_config(cfg: int, seed: int = 0, batch: int = None):
         raise ValueError("cfg must be 1..5")
     if batch is not None:
         B = batch
-    occ = gen(B, *shape, seed=seed)
+    occ = gen(B, *shape, seed=seed) if p is None else gen(B, *shape, p=p, seed=seed)
     idx, z_idx, z_ptr = _csr_from_occupancy(occ)
     return {"indices": idx, "z_idx": z_idx, "z_ptr": z_ptr,
             "spatial_shape": list(shape), "batch": B}
+
+
+def config2_with_voxels(voxels: int, seed: int = 0):
+    """Configuration 2's generator with its column occupancy raised (or lowered) until the scan holds about
+    ``voxels`` active voxels (within 0.5 %): -> (dict as make_config, occupancy used)."""
+    p = 0.5
+    d = make_config(2, seed=seed, p=p)
+    for _ in range(6):
+        n = int(d["z_idx"].shape[0])
+        if abs(n - voxels) <= 0.005 * voxels:
+            break
+        p = min(max(p * voxels / max(n, 1), 0.01), 1.0)
+        d = make_config(2, seed=seed, p=p)
+    return d, p
 
 
 def encoder_stack(in_channels: int = 16, widths=(16, 32, 64, 64), seed: int = 0, neighbours: float = 8.0):
