@@ -264,6 +264,33 @@ def configs_ms(torch, seed, iters):
         r["fwd_TFLOPs"] = 2.0 * P * ic * oc / r["fwd_us"] / 1e6
         out[name] = r
 
+    def run_refbench(name, subm, batch):
+        """The reference author's benchmark shapes (test/bench_conv.py:131-133, test/Untitled.ipynb): grid
+        [64, 512, 512] (512 bins on the compressed axis), 64 -> 64 fp16, real scans voxelised as the reference does."""
+        import numpy as np
+        import sphconv_amd as sphconv
+        from sphconv_amd.synth import lidar_scan_batch
+        path = os.path.join(ROOT, "tests", "golden", "kitti_000000_reduced.bin")
+        if not os.path.exists(path):
+            return
+        shape = [64, 512, 512]
+        feature, indices = lidar_scan_batch(np.fromfile(path, dtype=np.float32), batch, shape, 64, dev)
+        x = sphconv.SparseConvTensor(feature, shape, batch, indices=indices)
+        torch.manual_seed(seed)
+        w = (torch.randn((27, 64, 64), device=dev) * (2.0 / (27 * 64)) ** 0.5).half()
+        if subm:
+            mk = lambda: RuleBook.build_subm(x.z_idx, x.z_ptr, batch, shape, [3, 3, 3])
+        else:
+            mk = lambda: RuleBook.build(x.z_idx, x.z_ptr, batch, shape, [32, 256, 256], [3, 3, 3], [2, 2, 2], [1, 1, 1])
+        book = mk()
+        n, m, P = int(x.feature.shape[0]), book.out_rows, book.num_pairs()
+        r = {"in_rows": n, "out_rows": m, "pairs": P, "channels": [64, 64], "dtype": "float16", "batch": batch,
+             "rules_us": 1e3 * event_ms(mk, iters, torch),
+             "fwd_us": 1e3 * event_ms(lambda: ext.rule_conv(x.feature, w, book, None, m), iters, torch)}
+        r["fwd_GBps"] = (n * 128 + m * 128 + 27 * 64 * 64 * 2 + 8 * P) / r["fwd_us"] / 1e3
+        r["fwd_TFLOPs"] = 2.0 * P * 64 * 64 / r["fwd_us"] / 1e6
+        out[name] = r
+
     run("config1_subm_16_16_f32", 1, 16, 16, torch.float32)
     run("config2_subm_32_32_f16", 2, 32, 32, torch.float16)
     run("headline_subm_64_64_f16", 2, 64, 64, torch.float16)
@@ -271,6 +298,8 @@ def configs_ms(torch, seed, iters):
     run("config5a_subm_64_64_i8_b8", 5, 64, 64, torch.int8)
     run("config5b_subm_64_64_f16_b8", 5, 64, 64, torch.float16)
     run("headline_grid_8_scans_subm_64_64_f16", 2, 64, 64, torch.float16, batch=8)
+    run_refbench("reference_bench_k3s2p1_64_64_f16_b8_grid_64x512x512", False, 8)
+    run_refbench("reference_notebook_subm_64_64_f16_b3_grid_64x512x512", True, 3)
     return out
 
 

@@ -108,6 +108,36 @@ def config2_with_voxels(voxels: int, seed: int = 0):
     return d, p
 
 
+def lidar_scan_batch(points, batch: int, shape_dwh=(64, 512, 512), channels: int = 64, device="cuda:0"):
+    """The reference's benchmark inputs (test/common.py:30-59, used by test/bench_conv.py:131-133): LiDAR scans
+    voxelised on a spherical grid of ``shape_dwh`` cells (two points per voxel, at most 24000 voxels, mean VFE),
+    merged into a batch, the four point channels repeated up to ``channels``.  ``points`` [m,4] float32 is ONE
+    scan; sample i of the batch is that scan turned by 2 i degrees about the vertical axis (the reference
+    cycles through four scan files).  -> (feature [N,channels] fp16, indices [N,4] int32 (b, d, w, h)) on
+    ``device``."""
+    import torch
+
+    from .datagen import merge_batch_torch
+    from .vfe import SimpleVoxel
+    from .voxelize import VoxelGeneratorV3
+    points = np.asarray(points, dtype=np.float32).reshape(-1, 4)
+    gen = VoxelGeneratorV3(None, [6, -40, -3, 70.4, 40, 1], [6, -45, 87.5, 70.4, 45, 100], 2, 24000,
+                           list(shape_dwh)[::-1], coord_system="spherical")
+    vfe = SimpleVoxel(4)
+    examples = []
+    for i in range(batch):
+        a = np.deg2rad(2.0 * i)
+        rot = points.copy()
+        rot[:, 0] = np.cos(a) * points[:, 0] - np.sin(a) * points[:, 1]
+        rot[:, 1] = np.sin(a) * points[:, 0] + np.cos(a) * points[:, 1]
+        res = gen.generate(torch.from_numpy(rot).to(device))
+        voxels = vfe(res["voxels"], res["num_points_per_voxel"], res["coordinates"])
+        examples.append({"voxels": voxels, "coordinates": res["coordinates"]})
+    ex = merge_batch_torch(examples)
+    feature = ex["voxels"].repeat((1, (channels + 3) // 4))[:, :channels]
+    return feature.half().contiguous(), ex["coordinates"].int().contiguous()
+
+
 def encoder_stack(in_channels: int = 16, widths=(16, 32, 64, 64), seed: int = 0, neighbours: float = 8.0):
     """The four-stage middle encoder of benchmark configuration 4 as a ``Sequential``:
     per stage two submanifold 3x3x3 convolutions sharing one rule book, then a 3x3x3
