@@ -215,11 +215,13 @@ int sph_conv_apply(sph_dtype dt, const void *feature, int feature_rows, int kdim
  *   d_weight[k, ci, co] = sum over pairs (k, in, out) feature[in, ci] * d_out[out, co]
  * from a FORWARD book.  partial is fp32 scratch of
  * sph_wgrad_partial_elems(KV, iC, oC, rows) elements; the reduction over it is
- * done in fp32 in a fixed order.  d_weight has the element type dt. */
+ * done in fp32 in a fixed order.  d_weight [KV, iC, oC] has the element type dt, or is fp32
+ * when d_weight_f32 != 0 (16-bit features with an fp32 master weight: the sums over 1e5
+ * pairs need not be rounded to, or overflow, a 16-bit type). */
 size_t sph_wgrad_partial_elems(int KV, int iC, int oC, int out_rows);
 int sph_conv_wgrad(sph_dtype dt, const void *feature, int in_rows, int iC, const void *d_out,
                    int oC, const sph_book *fwd_book, float *partial, void *d_weight,
-                   void *stream);
+                   int d_weight_f32, void *stream);
 
 /* ---- tensor construction / densify (tensor.cu) ------------------------- */
 

@@ -42,7 +42,7 @@ class Epilogue(C.Structure):
 
 
 _lib = None
-ABI_VERSION = 4       # sph_abi_version() of the library these signatures describe
+ABI_VERSION = 5       # sph_abi_version() of the library these signatures describe
 
 _I, _P, _L, _Z = C.c_int, C.c_void_p, C.c_long, C.c_size_t
 _SIGNATURES = {
@@ -68,7 +68,7 @@ _SIGNATURES = {
     "sph_weight_pack": (_I, [_I, _P, _I, _I, _I, _L, _L, _L, _P, _P]),
     "sph_conv_apply": (_I, [_I, _P, _I, _I, _P, _I, C.POINTER(Book), C.POINTER(Epilogue), _P, _P]),
     "sph_wgrad_partial_elems": (_Z, [_I, _I, _I, _I]),
-    "sph_conv_wgrad": (_I, [_I, _P, _I, _I, _P, _I, C.POINTER(Book), _P, _P, _P]),
+    "sph_conv_wgrad": (_I, [_I, _P, _I, _I, _P, _I, C.POINTER(Book), _P, _P, _I, _P]),
     "sph_init_tensor_workspace": (_Z, [_I, _I, _I, _I, _I]),
     "sph_init_tensor": (_I, [_P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _Z, _P]),
     "sph_permute_rows": (_I, [_P, _P, _I, _I, _I, _P, _P]),

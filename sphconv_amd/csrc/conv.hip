@@ -1092,9 +1092,8 @@ __global__ __launch_bounds__(kWgThreads) void wgrad_kernel(WgradArgs a)
     }
 }
 
-template <sph_dtype DT>
-__global__ void wgrad_reduce_kernel(const float *partial, int KV, int nchunk, int per_k,
-                                    typename Traits<DT>::elem *dw)
+template <typename OUT>
+__global__ void wgrad_reduce_kernel(const float *partial, int KV, int nchunk, int per_k, OUT *dw)
 {
     long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (long)KV * per_k) return;
@@ -1102,7 +1101,7 @@ __global__ void wgrad_reduce_kernel(const float *partial, int KV, int nchunk, in
     const float *p = partial + (long)k * nchunk * per_k + e;
     float s = 0.f;
     for (int c = 0; c < nchunk; c++) s += p[(long)c * per_k];
-    dw[i] = (typename Traits<DT>::elem)s;
+    dw[i] = (OUT)s;
 }
 
 // ---------------------------------------------------------------------------
@@ -1415,10 +1414,9 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
 // slots are read as they were written; a workgroup covers 32 consecutive items, its 8 groups of
 // 32 threads each add every 8th slot (up to sixteen loads in flight), and the 8 sub-sums are added in a
 // fixed order.
-template <sph_dtype DT>
+template <typename OUT>
 __global__ __launch_bounds__(256) void wgrad_slot_reduce_kernel(const float *partial, const int *flags, int slots_per_k,
-                                                                int iC, int oC, int mi_tiles, int ni_tiles,
-                                                                typename Traits<DT>::elem *dw)
+                                                                int iC, int oC, int mi_tiles, int ni_tiles, OUT *dw)
 {
     __shared__ float4v s_sum[8][32];
     __shared__ unsigned long long s_flags[16];
@@ -1471,7 +1469,7 @@ __global__ __launch_bounds__(256) void wgrad_slot_reduce_kernel(const float *par
         if (co < oC) {
 #pragma unroll
             for (int v = 0; v < 4; v++)
-                if (ci + v < iC) dw[((long)k * iC + ci + v) * oC + co] = (typename Traits<DT>::elem)r[v];
+                if (ci + v < iC) dw[((long)k * iC + ci + v) * oC + co] = (OUT)r[v];
         }
     }
 }
@@ -1632,7 +1630,7 @@ inline bool wgrad_wave_ok(sph_dtype dt, int iC, int oC)
 }
 
 template <sph_dtype DT>
-int launch_wgrad(const WgradArgs &a0, void *dw, hipStream_t st)
+int launch_wgrad(const WgradArgs &a0, void *dw, bool f32_out, hipStream_t st)
 {
     typedef typename Traits<DT>::elem elem;
     const int KV = a0.book.KV;
@@ -1671,8 +1669,12 @@ int launch_wgrad(const WgradArgs &a0, void *dw, hipStream_t st)
 #undef SPH_WGRAD_CASE
         rc = sph_check_launch("sph_conv_wgrad");
         if (rc) return rc;
-        hipLaunchKernelGGL(wgrad_slot_reduce_kernel<DT>, dim3((unsigned)(mi * ni * 2), sb, KV), dim3(256), 0, st,
-                           a.partial, a.flags, a.nchunk * a.nslice, a.iC, a.oC, mi, ni, (elem *)dw);
+        if (f32_out)
+            hipLaunchKernelGGL(wgrad_slot_reduce_kernel<float>, dim3((unsigned)(mi * ni * 2), sb, KV), dim3(256), 0, st,
+                               a.partial, a.flags, a.nchunk * a.nslice, a.iC, a.oC, mi, ni, (float *)dw);
+        else
+            hipLaunchKernelGGL(wgrad_slot_reduce_kernel<elem>, dim3((unsigned)(mi * ni * 2), sb, KV), dim3(256), 0, st,
+                               a.partial, a.flags, a.nchunk * a.nslice, a.iC, a.oC, mi, ni, (elem *)dw);
         return sph_check_launch("sph_conv_wgrad(reduce)");
     }
     const WgradArgs &a = a0;
@@ -1682,8 +1684,12 @@ int launch_wgrad(const WgradArgs &a0, void *dw, hipStream_t st)
     hipLaunchKernelGGL(wgrad_kernel<DT>, dim3(KV * a.nchunk), dim3(kWgThreads), lds, st, a);
     int rc = sph_check_launch("sph_conv_wgrad");
     if (rc) return rc;
-    hipLaunchKernelGGL(wgrad_reduce_kernel<DT>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                       a.partial, KV, a.nchunk, per_k, (elem *)dw);
+    if (f32_out)
+        hipLaunchKernelGGL(wgrad_reduce_kernel<float>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                           a.partial, KV, a.nchunk, per_k, (float *)dw);
+    else
+        hipLaunchKernelGGL(wgrad_reduce_kernel<elem>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                           a.partial, KV, a.nchunk, per_k, (elem *)dw);
     return sph_check_launch("sph_conv_wgrad(reduce)");
 }
 
@@ -1770,7 +1776,8 @@ SPH_EXPORT size_t sph_wgrad_partial_elems(int KV, int iC, int oC, int out_rows)
 }
 
 SPH_EXPORT int sph_conv_wgrad(sph_dtype dt, const void *feature, int in_rows, int iC, const void *d_out,
-                              int oC, const sph_book *fwd_book, float *partial, void *d_weight, void *stream)
+                              int oC, const sph_book *fwd_book, float *partial, void *d_weight, int d_weight_f32,
+                              void *stream)
 {
     SPH_REQUIRE(book_ok(fwd_book) && book_has_groups(fwd_book), SPH_ERR_ARG, "sph_conv_wgrad: bad book (it must hold its groups)");
     SPH_REQUIRE(partial && d_weight, SPH_ERR_ARG, "sph_conv_wgrad: null pointer");
@@ -1797,8 +1804,8 @@ SPH_EXPORT int sph_conv_wgrad(sph_dtype dt, const void *feature, int in_rows, in
     a.nslice = kWsSlices;
     hipStream_t st = (hipStream_t)stream;
     switch (dt) {
-    case SPH_F32: return launch_wgrad<SPH_F32>(a, d_weight, st);
-    case SPH_F16: return launch_wgrad<SPH_F16>(a, d_weight, st);
-    default: return launch_wgrad<SPH_BF16>(a, d_weight, st);
+    case SPH_F32: return launch_wgrad<SPH_F32>(a, d_weight, true, st);
+    case SPH_F16: return launch_wgrad<SPH_F16>(a, d_weight, d_weight_f32 != 0, st);
+    default: return launch_wgrad<SPH_BF16>(a, d_weight, d_weight_f32 != 0, st);
     }
 }

@@ -15,6 +15,10 @@ class ConvFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, feature, weight, rules, rule_size, tile_grid_shape: List[int], outNNZ: int, packed=None):
+        if (ctx.needs_input_grad[0] or ctx.needs_input_grad[1]) and weight.shape[1] > ext.MAX_TRAIN_CHANNELS:
+            # forward alone takes up to 256 input channels; say so here, not from inside backward()
+            raise ext.L.SphconvError("training takes 1..%d input channels (forward alone up to %d), got %d"
+                                     % (ext.MAX_TRAIN_CHANNELS, ext.MAX_FORWARD_IN_CHANNELS, weight.shape[1]))
         book = rules if isinstance(rules, RuleBook) else RuleBook.from_padded(
             rules, rule_size, feature.shape[0], int(outNNZ))
         ctx.save_for_backward(feature, weight)
@@ -41,7 +45,10 @@ class ConvFunction(torch.autograd.Function):
             packed = ext._packed_weight(w, True, reverse)
             d_feature = ext._apply(d_out, packed, w.shape[2], w.shape[1], buf)
         if ctx.needs_input_grad[1]:
-            d_weight = ext.rule_conv_d_weight(feature, d_out, book, None).to(weight.dtype)
+            # an fp32 master weight gets its gradient straight from the fp32 reduction, not through a 16-bit type
+            want_f32 = weight.dtype == torch.float32
+            d_weight = ext.rule_conv_d_weight(feature, d_out, book, None,
+                                              torch.float32 if want_f32 else None).to(weight.dtype)
         return d_feature, d_weight, None, None, None, None, None
 
 

@@ -22,6 +22,12 @@ import torch
 from . import _lib as L
 from .rulebook import RuleBook
 
+# channel limits of the kernels: forward contracts over up to 256 input channels into up to 128 output
+# channels; dgrad writes iC columns and wgrad keeps an iC x oC tile per offset, so training needs both <= 128
+MAX_FORWARD_IN_CHANNELS = 256
+MAX_OUT_CHANNELS = 128
+MAX_TRAIN_CHANNELS = 128
+
 __version__ = "hip-gfx950"
 
 # Packed copies of weights seen while no gradient is being recorded (inference): one per (weight storage,
@@ -287,8 +293,10 @@ def rule_conv_d_feature(feature: torch.Tensor, weight: torch.Tensor, rules, rule
     return _apply(feature, packed, weight.shape[1], weight.shape[2], buf)
 
 
-def rule_conv_d_weight(feature: torch.Tensor, d_featureOut: torch.Tensor, rules, ruleSize) -> torch.Tensor:
-    """rule_conv.cu:469-518 -> d_weight [KV,iC,oC], reduced in fp32."""
+def rule_conv_d_weight(feature: torch.Tensor, d_featureOut: torch.Tensor, rules, ruleSize,
+                       out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """rule_conv.cu:469-518 -> d_weight [KV,iC,oC], reduced in fp32 and stored in the features' type, or in
+    float32 with ``out_dtype=torch.float32`` (16-bit features with an fp32 master weight)."""
     book = _as_book(rules, ruleSize, feature.shape[0], d_featureOut.shape[0])
     feature = feature.contiguous()
     d_out = d_featureOut.contiguous()
@@ -298,10 +306,13 @@ def rule_conv_d_weight(feature: torch.Tensor, d_featureOut: torch.Tensor, rules,
     ic, oc = feature.shape[1], d_out.shape[1]
     n = lib.sph_wgrad_partial_elems(book.kv, ic, oc, book.out_rows)
     partial = torch.empty(max(n, 1), dtype=torch.float32, device=feature.device)
-    dw = torch.empty((book.kv, ic, oc), dtype=feature.dtype, device=feature.device)
+    if out_dtype not in (None, feature.dtype, torch.float32):
+        raise L.SphconvError("d_weight comes in the features' type or in float32, not %s" % out_dtype)
+    f32 = out_dtype == torch.float32
+    dw = torch.empty((book.kv, ic, oc), dtype=torch.float32 if f32 else feature.dtype, device=feature.device)
     b = book.grouped().struct()
     L.check(lib.sph_conv_wgrad(L.dtype_code(feature.dtype), L.ptr(feature), feature.shape[0], ic,
-                               L.ptr(d_out), oc, C.byref(b), L.ptr(partial), L.ptr(dw), L.stream()))
+                               L.ptr(d_out), oc, C.byref(b), L.ptr(partial), L.ptr(dw), int(f32), L.stream()))
     return dw
 
 

@@ -278,6 +278,12 @@ def test_wgrad_channel_blocks_and_chunks(dtype, ic, oc, subm):
     # run-to-run determinism (fixed summation order)
     again = ext.rule_conv_d_weight(feat.to(G.DEV), g.to(G.DEV), book, None)
     assert torch.equal(again, d_w)
+    # the same reduction stored as fp32 (an fp32 master weight): no rounding to the storage type, and rounding
+    # it afterwards gives the typed result bit for bit
+    wide = ext.rule_conv_d_weight(feat.to(G.DEV), g.to(G.DEV), book, None, torch.float32)
+    assert wide.dtype == torch.float32
+    assert torch.equal(wide.to(dtype), d_w)
+    assert (np.abs(wide.double().cpu().numpy() - ref) <= 1e-5 * mag + 1e-6).all()
 
 
 def test_fused_epilogue_scale_shift_relu():
@@ -644,3 +650,25 @@ def test_wgrad_many_slots_equals_sum_over_samples():
     # every part was rounded to fp16 once, the whole once; the sums run over up to 2.2 M products (centre offset)
     scale = float(whole.abs().max())
     assert float((whole - parts).abs().max()) <= 2.0 ** -9 * scale * np.sqrt(B) + 1e-2
+
+
+def test_fp32_master_weight_gets_an_fp32_gradient():
+    """fp16 features with an fp32 weight (mixed-precision training): the weight's gradient is the fp32
+    reduction itself, never rounded to, or overflowing in, fp16."""
+    from sphconv_amd.functional import ConvFunction
+    case = _random_case(77, True)
+    rng = np.random.default_rng(5)
+    n = case["sidx"].shape[0]
+    # values whose sums over a neighbourhood leave fp16's range: a 16-bit d_weight would be inf
+    feat = G.t(rng.standard_normal((n, 16)).astype(np.float32) * 60).half().requires_grad_(True)
+    w = G.t(_weights(rng, 27, 16, 32)).requires_grad_(True)
+    out = ConvFunction.apply(feat, w, case["book"], None, [1, 1], n)
+    assert out.dtype == torch.float16
+    up = G.t(rng.standard_normal((n, 32)).astype(np.float32) * 60).half()
+    out.backward(up)
+    assert w.grad.dtype == torch.float32 and torch.isfinite(w.grad).all()
+    wide = ext.rule_conv_d_weight(feat.detach(), up, case["book"], None, torch.float32)
+    assert torch.equal(w.grad, wide)
+    assert wide.abs().max() > 65504          # the case does leave fp16's range
+    narrow = ext.rule_conv_d_weight(feat.detach(), up, case["book"], None)
+    assert torch.isinf(narrow).any()

@@ -86,3 +86,15 @@ def test_bench_refuses_more_than_one_gpu():
     import sys
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode == 2 and "ONE GPU" in r.stderr and r.stdout == ""
+
+
+def test_training_channel_limit_is_reported_before_forward():
+    """Forward takes up to 256 input channels, dgrad/wgrad up to 128: a module that wants gradients says so
+    when it is called, not from inside backward()."""
+    import torch
+    import sphconv_amd
+    from sphconv_amd.functional import ConvFunction
+    feature = torch.zeros((4, 192), requires_grad=True)
+    weight = torch.zeros((27, 192, 32), requires_grad=True)
+    with pytest.raises(sphconv_amd.SphconvError, match="training takes 1..128 input channels"):
+        ConvFunction.apply(feature, weight, None, None, [1, 1], 4)
