@@ -29,8 +29,8 @@
 #include <cstring>
 
 #include <rocprim/device/device_radix_sort.hpp>
-#include <rocprim/device/device_scan.hpp>
-#include <rocprim/functional.hpp>
+
+#include "scan.h"
 
 namespace {
 
@@ -47,29 +47,22 @@ inline int key_bits(long cells)
     return b;
 }
 
-// temporary storage rocPRIM asks for (sort of n pairs, scan of ncol ints); 0 on error
+// temporary storage of the sort of n pairs (what rocPRIM asks for) and of the scan of ncol ints, which share
+// one area; 0 on error
 inline size_t library_temp_bytes(int n, int ncol, long cells)
 {
-    size_t sort_bytes = 0, scan_bytes = 0;
+    size_t sort_bytes = 0;
     hipError_t e = rocprim::radix_sort_pairs(nullptr, sort_bytes, (const uint64_t *)nullptr, (uint64_t *)nullptr,
                                              (const int32_t *)nullptr, (int32_t *)nullptr, (size_t)(n > 0 ? n : 1), 0,
                                              key_bits(cells), (hipStream_t)0);
     if (e != hipSuccess) return 0;
-    e = rocprim::inclusive_scan(nullptr, scan_bytes, (int32_t *)nullptr, (int32_t *)nullptr, (size_t)(ncol > 0 ? ncol : 1),
-                                rocprim::maximum<int32_t>(), (hipStream_t)0);
-    if (e != hipSuccess) return 0;
+    const size_t scan_bytes = sph_scan::state_bytes(ncol);
     return (sort_bytes > scan_bytes ? sort_bytes : scan_bytes) + 256;
 }
 
 constexpr int kRankMaxDepth = 128; // S2 up to which rows are ranked inside their column instead of sorted
 
-inline size_t sum_scan_bytes(int ncol)
-{
-    size_t b = 0;
-    hipError_t e = rocprim::inclusive_scan(nullptr, b, (int32_t *)nullptr, (int32_t *)nullptr, (size_t)(ncol > 0 ? ncol : 1),
-                                           rocprim::plus<int32_t>(), (hipStream_t)0);
-    return e == hipSuccess ? b + 256 : 0;
-}
+inline size_t sum_scan_bytes(int ncol) { return sph_scan::state_bytes(ncol); }
 
 struct RankLayout {
     size_t slot, seg_z, seg_row, temp, temp_bytes, total;
@@ -232,8 +225,7 @@ static int init_tensor_by_rank(const int32_t *indices, int n, int B, int S0, int
     hipLaunchKernelGGL(coo_count_kernel, grid, block, 0, st, indices, n, B, S0, S1, S2, z_ptr, slot, status);
     rc = sph_check_launch("sph_init_tensor(count)");
     if (rc) return rc;
-    size_t temp_bytes = l.temp_bytes;
-    hipError_t e = rocprim::inclusive_scan(ws + l.temp, temp_bytes, z_ptr, z_ptr, (size_t)ncol, rocprim::plus<int32_t>(), st);
+    hipError_t e = sph_scan::launch<sph_scan::Plus, true>(z_ptr, z_ptr, ncol, ws + l.temp, 0, st);
     if (e != hipSuccess) {
         sph_set_error("sph_init_tensor: scan: %s", hipGetErrorString(e));
         return SPH_ERR_LAUNCH;
@@ -288,8 +280,7 @@ SPH_EXPORT int sph_init_tensor(const int32_t *indices, int n, int B, int S0, int
                        (const int32_t *)vals_out, n, S2, ncol, z_idx, z_ptr, permutation, status);
     rc = sph_check_launch("sph_init_tensor(finish)");
     if (rc) return rc;
-    temp_bytes = l.temp_bytes;
-    e = rocprim::inclusive_scan(ws + l.temp, temp_bytes, z_ptr, z_ptr, (size_t)ncol, rocprim::maximum<int32_t>(), st);
+    e = sph_scan::launch<sph_scan::Max, true>(z_ptr, z_ptr, ncol, ws + l.temp, 0, st);
     if (e != hipSuccess) {
         sph_set_error("sph_init_tensor: scan: %s", hipGetErrorString(e));
         return SPH_ERR_LAUNCH;

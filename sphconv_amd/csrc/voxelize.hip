@@ -22,8 +22,8 @@
 #include <cstring>
 
 #include <rocprim/device/device_radix_sort.hpp>
-#include <rocprim/device/device_scan.hpp>
-#include <rocprim/functional.hpp>
+
+#include "scan.h"
 
 namespace {
 
@@ -186,18 +186,13 @@ inline VoxLayout vox_layout(int n, unsigned long long cells)
     l.start = o; o += al256(nn * 4);
     l.stop = o; o += 256;
     l.temp = o;
-    size_t sort_b = 0, scan_b = 0, scan2_b = 0;
+    // the sort's temporary storage (what rocPRIM asks for) and the scans' state share one area
+    size_t sort_b = 0;
     hipError_t e = rocprim::radix_sort_pairs(nullptr, sort_b, (const uint64_t *)nullptr, (uint64_t *)nullptr,
                                              (const int32_t *)nullptr, (int32_t *)nullptr, nn, 0, bits_for(cells),
                                              (hipStream_t)0);
-    if (e == hipSuccess)
-        e = rocprim::exclusive_scan(nullptr, scan_b, (int32_t *)nullptr, (int32_t *)nullptr, 0, nn, rocprim::plus<int32_t>(),
-                                    (hipStream_t)0);
-    if (e == hipSuccess)
-        e = rocprim::inclusive_scan(nullptr, scan2_b, (int32_t *)nullptr, (int32_t *)nullptr, nn, rocprim::maximum<int32_t>(),
-                                    (hipStream_t)0);
-    size_t t = sort_b > scan_b ? sort_b : scan_b;
-    if (scan2_b > t) t = scan2_b;
+    const size_t scan_b = sph_scan::state_bytes((long)nn);
+    const size_t t = sort_b > scan_b ? sort_b : scan_b;
     l.temp_bytes = e == hipSuccess ? t + 256 : 0;
     l.total = l.temp_bytes ? o + al256(l.temp_bytes) : 0;
     return l;
@@ -263,13 +258,9 @@ SPH_EXPORT int sph_points_to_voxel(const float *points, int n, int nfeat, int sy
     if (e == hipSuccess) {
         hipLaunchKernelGGL(vox_head_kernel, dim3(blocks(n)), dim3(256), 0, st, (const uint64_t *)keys_out,
                            (const int32_t *)vals_out, n, (uint64_t)q.cells, mark, start_in);
-        tb = l.temp_bytes;
-        e = rocprim::exclusive_scan(ws + l.temp, tb, mark, vid, 0, (size_t)n, rocprim::plus<int32_t>(), st);
+        e = sph_scan::launch<sph_scan::Plus, false>(mark, vid, n, ws + l.temp, 0, st);
     }
-    if (e == hipSuccess) {
-        tb = l.temp_bytes;
-        e = rocprim::inclusive_scan(ws + l.temp, tb, start_in, start, (size_t)n, rocprim::maximum<int32_t>(), st);
-    }
+    if (e == hipSuccess) e = sph_scan::launch<sph_scan::Max, true>(start_in, start, n, ws + l.temp, 0, st);
     if (e != hipSuccess) {
         sph_set_error("sph_points_to_voxel: sort/scan: %s", hipGetErrorString(e));
         return SPH_ERR_LAUNCH;

@@ -201,11 +201,13 @@ def test_extension_functions_match_reference_signatures():
 
 @pytest.mark.parametrize("B,shape,n", [(1, (64, 512, 32), 40000), (3, (7, 5, 3), 50), (2, (2048, 2048, 1024), 3000),
                                        (1, (4, 4, 4), 0), (1, (1, 1, 1), 1), (2, (8, 8, 64), 6000),
-                                       (1, (16, 16, 128), 20000), (1, (16, 16, 129), 20000), (1, (3, 3, 200), 0)])
+                                       (1, (16, 16, 128), 20000), (1, (16, 16, 129), 20000), (1, (3, 3, 200), 0),
+                                       (1, (1024, 1024, 16), 150000), (2, (512, 300, 130), 90000)])
 def test_init_tensor_sizes(B, shape, n):
     """COO -> compressed layout at sizes that need more than 32 key bits, one cell, no voxel
-    at all, long fibers, and either side of the depth (128 bins) at which rows are sorted instead of
-    ranked inside their column; checked against the oracle and against the defining invariants."""
+    at all, long fibers, either side of the depth (128 bins) at which rows are sorted instead of
+    ranked inside their column, and column counts whose scan looks back over more than 64 workgroups
+    (sum scan: 1M columns; max scan: 307k); checked against the oracle and against the defining invariants."""
     rng = np.random.default_rng(B * 1000 + n)
     cells = B * shape[0] * shape[1] * shape[2]
     lin = np.unique(rng.integers(0, cells, size=n, dtype=np.int64))[:n] if n else np.zeros(0, np.int64)

@@ -64,6 +64,25 @@ def test_kitti_scan(system, grid, max_points, max_voxels, append_mode):
         _compare({k: v for k, v in res.items() if k != "cells"}, want)
 
 
+def test_many_points_scan_over_many_workgroups():
+    """Eight jittered copies of the reference's scan (about 150 000 points): the voxel numbering and the
+    first-point search scan arrays of more than 64 workgroups' worth of elements.  Integer part on the
+    oracle's cells, bit-exact."""
+    base = np.fromfile(KITTI, dtype=np.float32).reshape(-1, 4)
+    rng = np.random.default_rng(3)
+    pts = np.concatenate([base + rng.normal(0, 0.05, base.shape).astype(np.float32) for _ in range(8)])
+    assert pts.shape[0] > 64 * 2048
+    grid, max_points, max_voxels = [512, 512, 64], 3, 200000
+    sp, rg = O.system_transform(pts, RANGE, SRANGE, "spherical")
+    coor, ok, _ = O.voxel_cells(sp, rg, grid)
+    cells = np.where(ok, (coor[:, 0] * grid[1] + coor[:, 1]) * grid[0] + coor[:, 2], -1)
+    want = O.voxelize_cells(pts, sp, coor, ok, max_points, max_voxels, 0)
+    res = points_to_voxel_v2(pts, None, RANGE, SRANGE, None, max_points, max_voxels, resolution_HWD=grid,
+                             coord_system="spherical", append_mode=0, cells=torch.tensor(cells))
+    _compare(res, want)
+    assert want["voxel_num"] > 30000
+
+
 def test_small_and_degenerate_inputs():
     pts = np.array([[20, 1, 0.2, 0.5], [20, 1, 0.2, 0.6], [0, 0, 3, 0.1], [0, 0, 0, 0.2], [1e3, 5, 1, 0.3],
                     [30, -2, -1, 0.4], [20, 1, 0.2, 0.7]], np.float32)
