@@ -66,6 +66,11 @@ def parse():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 256 MiB device-to-device copies (a kernel of known HBM traffic, "
                          "to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+    ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: read the counter_collection.csv files of two `rocprofv3 --pmc FETCH_SIZE` / "
+                         "`--pmc WRITE_SIZE` runs of `bench.py --copy-calibration --streams 1 --no-cpu-baseline` and "
+                         "write profiles/hbm_traffic.json (HBM bytes per launch of the two kernels of the step at "
+                         "both scan sizes, each counter scaled by what it reads for the 256 MiB copies)")
     return ap.parse_args()
 
 
@@ -332,6 +337,68 @@ def recorded_traffic(kernel_key, voxels, seed):
     return None
 
 
+COPY_BYTES = 256 << 20      # bytes read (and written) by one --copy-calibration copy
+COPY_COUNT = 3
+
+
+def record_traffic(fetch_csv, write_csv, seed, voxels):
+    """profiles/hbm_traffic.json from two counter runs.  A kernel's dispatches are told apart by name and grid
+    size (the grid follows from the scan's tile count); the counters are KiB per dispatch, and each is scaled by
+    total bytes of the calibration copies / what the counter summed to over the copy dispatches."""
+    import csv
+    from collections import defaultdict
+    from sphconv_amd.synth import config2_with_voxels, make_config
+
+    def load(path, counter):
+        per = defaultdict(list)
+        copy_sum = 0.0
+        with open(path, newline="") as f:
+            for r in csv.DictReader(f):
+                if r["Counter_Name"] != counter:
+                    continue
+                name, v = r["Kernel_Name"], float(r["Counter_Value"])
+                if "copyBuffer" in name and v >= 16384:    # the calibration copies, not torch's small tensor clones
+                    copy_sum += v
+                per[(name, int(r["Grid_Size"]))].append(v)
+        if copy_sum <= 0:
+            raise SystemExit("%s: no copy dispatches (run bench.py with --copy-calibration)" % path)
+        factor = COPY_COUNT * COPY_BYTES / 1024.0 / copy_sum
+        return per, factor
+
+    fetch, f_fetch = load(fetch_csv, "FETCH_SIZE")
+    write, f_write = load(write_csv, "WRITE_SIZE")
+    sizes = [int(make_config(2, seed=seed)["z_idx"].shape[0])]
+    if voxels > 0:
+        sizes.append(int(config2_with_voxels(voxels, seed=seed)[0]["z_idx"].shape[0]))
+    kernels = []
+    for n in sizes:
+        blocks = ((n + 127) // 128 + 7) // 8 * 8        # tiles, rounded up to whole rounds over the 8 XCDs
+        wanted = {"conv": ("conv_wave_kernel", lambda g: g == blocks * 64),
+                  # the step's launch: one workgroup of 256 threads per tile, then the ones that pack the weight
+                  # (the per-kernel section also launches it without them)
+                  "rules": ("build_book_kernel<false>", lambda g: blocks * 256 < g <= (blocks + 512) * 256)}
+        for key, (pat, grid_ok) in wanted.items():
+            def mean(per):
+                vals = [v for (name, g), vs in per.items() if pat in name and grid_ok(g) for v in vs]
+                if not vals:
+                    raise SystemExit("no dispatch of %s for a scan of %d voxels in the counter files" % (pat, n))
+                return sum(vals) / len(vals), len(vals)
+            (fk, nf), (wk, nw) = mean(fetch), mean(write)
+            kernels.append({"key": key, "voxels": n, "kernel": pat, "dispatches": [nf, nw],
+                            "fetch_kib": round(fk, 1), "write_kib": round(wk, 1),
+                            "hbm_bytes": int(round((fk * f_fetch + wk * f_write) * 1024))})
+    rec = {"sources_sha256": kernel_sources_digest(), "seed": seed,
+           "fetch_scale": round(f_fetch, 4), "write_scale": round(f_write, 4),
+           "calibration": "%d device copies of %d MiB (--copy-calibration): bytes copied / counter sum over their "
+                          "dispatches" % (COPY_COUNT, COPY_BYTES >> 20),
+           "kernels": kernels}
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    with open(path, "w") as f:
+        json.dump(rec, f, indent=1)
+        f.write("\n")
+    print(json.dumps(rec))
+
+
 class Workload:
     """One scan size of the benchmark: `copies` device-resident copies of the scan (index arrays and
     features in separate allocations, so that the timed steps walk through more memory than the 256 MB
@@ -392,8 +459,7 @@ class Workload:
             for i in range(steps):
                 k = (r * steps + i) % len(self.scans)
                 last = (pipe.submit(*self.scans[k], wait_inputs=False), k)   # inputs are resident and complete
-            pipe.synchronize()
-            torch.cuda.synchronize()
+            torch.cuda.synchronize()      # every stream of the device (one wait, not one per stream)
             times.append((time.perf_counter() - t0) / steps * 1e3)
         (out_p, _slot), k = last
         _, out = self.step(k)
@@ -462,6 +528,9 @@ def main():
         print("bench.py: this build runs the hot path on ONE GPU; --gpus %d is not supported "
               "(no collectives are part of this path)" % args.gpus, file=sys.stderr)
         sys.exit(2)
+    if args.record_traffic:
+        record_traffic(args.record_traffic[0], args.record_traffic[1], args.seed, args.voxels)
+        return
     import numpy as np
     import torch
 
@@ -477,9 +546,9 @@ def main():
     d = make_config(2, seed=args.seed)
 
     if args.copy_calibration:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        src = torch.empty(COPY_BYTES, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
-        for _ in range(3):
+        for _ in range(COPY_COUNT):
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
