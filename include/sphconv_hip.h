@@ -131,16 +131,15 @@ int sph_rules_build_pack(const int32_t *z_idx, const int32_t *z_ptr, int in_rows
 
 /* Replaces the output-coordinate half of get_rules (rules.cu:417-443, 461-462: prepareGridKernel, two
  * cumsums, roll/index_put/add and the device->host read), in two steps because the caller must size oz_idx:
- *  1. sph_outcoords_count: ONE launch counts every output column's active bins and scans the counts
- *     (single pass: workgroups of 64 columns look back over their predecessors' sums) into oz_ptr
+ *  1. sph_outcoords_count: one kernel counts every output column's active bins and scans the counts
+ *     (single pass: workgroups of 64 to 512 columns look back over their predecessors' sums) into oz_ptr
  *     (inclusive), and writes the number of output rows to *total_dev (null: not written; it is also the
  *     last element of oz_ptr).  total_dev is any address the GPU can write: device memory, or pinned host
  *     memory (hipHostMalloc) that the host reads after synchronising the stream, without a copy.
- *     `scratch`: 8-byte aligned device memory of sph_outcoords_scratch_ints(g) int32; its first
- *     sph_outcoords_state_ints(g) entries hold the state of the scan across workgroups and MUST BE ZERO
- *     when the call is enqueued; the launch leaves them zero again, so a scratch that was zeroed once
- *     serves any number of calls one after another (calls that overlap on one scratch race).  Behind the
- *     state, when O[2] <= 64, each column's 64-bit mask of active bins is kept for step 2.
+ *     `scratch`: 8-byte aligned device memory of sph_outcoords_scratch_ints(g) int32, contents arbitrary;
+ *     its first sph_outcoords_state_ints(g) entries hold the state of the scan across workgroups, which a
+ *     small fill kernel in front of the count kernel clears (calls that overlap on one scratch race).
+ *     Behind the state, when O[2] <= 64, each column's 64-bit mask of active bins is kept for step 2.
  *  2. once the caller knows the total: sph_outcoords_fill, given the same scratch and oz_ptr, writes
  *     oz_idx (ascending within a column).
  * sph_outcoords_blocks(g) = ceil(columns / 256), the grid of the fill kernel. */

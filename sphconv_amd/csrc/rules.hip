@@ -589,7 +589,11 @@ __device__ unsigned long long column_mask(const OutArgs &a, int b, int o0, int o
 }
 
 constexpr int kColLanes = 16;                    // lanes that share one output column
-constexpr int kCountCols = 64;                   // output columns per workgroup of the count kernel
+#ifndef SPH_COUNT_COLS
+#define SPH_COUNT_COLS 64
+#endif
+constexpr int kCountCols = SPH_COUNT_COLS;       // output columns per workgroup of the count kernel (at most 64)
+static_assert(kCountCols <= kWave && (kCountCols & (kCountCols - 1)) == 0, "one wave scans a workgroup's counts");
 constexpr int kCountThreads = kCountCols * kColLanes;
 
 // OR over the 16 lanes of a column group (all 16 are active together).
@@ -604,9 +608,11 @@ __device__ __forceinline__ unsigned long long or_reduce16(unsigned long long m)
     return ((unsigned long long)hi << 32) | lo;
 }
 
-// State of the scan across workgroups, at the head of the caller's scratch: a ticket counter, a counter
-// of finished workgroups and one 64-bit status word per workgroup (flag in the two top bits, value in
-// the low 32).  All of it is zero between launches: the last workgroup to finish clears it.
+// State of the scan across workgroups, at the head of the caller's scratch: a ticket counter (and a spare
+// word that keeps the status words 8-byte aligned) and one 64-bit status word per workgroup (flag in the two
+// top bits, value in the low 32).  A fill kernel clears it in front of every count launch: a counter of
+// finished workgroups, by which the last one could clear it instead, costs every workgroup a second atomic on
+// one address, and those queue up behind one another across the XCDs.
 constexpr unsigned long long kScanAggregate = 1ull << 62; // value = sum of the workgroup's own counts
 constexpr unsigned long long kScanInclusive = 2ull << 62; // value = sum of all counts up to and including it
 __host__ __device__ inline int count_blocks(long ncol) { return (int)((ncol + kCountCols - 1) / kCountCols); }
@@ -623,52 +629,68 @@ __device__ __forceinline__ void status_store(unsigned long long *p, unsigned lon
 
 // Per-column counts and their inclusive scan (oz_ptr) in one launch.  16 lanes share an output column (one
 // input column (k0, k1) each, K0*K1 = 9 of them busy for a 3x3x3 kernel), so the fibers that reach a column
-// are walked side by side and small grids still fill the chip; a workgroup takes 64 columns.  Workgroups
-// number themselves by a ticket (so every predecessor of a workgroup is already running), publish the sum
-// of their counts, and look back over their predecessors' status words, 64 at a time, until they meet one
-// that already knows its inclusive prefix.  `masks` (O2 <= 64 only, else null) keeps each column's bin mask
-// for the fill kernel; `total` (may be null) receives the number of output rows.
+// are walked side by side and small grids still fill the chip; a workgroup takes `passes` batches of 64
+// consecutive columns (the launcher gives large grids several, so that a few hundred workgroups share the
+// ticket counter and the status words: with one batch each, 2048 workgroups spent most of the kernel queueing
+// for them).  Workgroups number themselves by a ticket (so every predecessor of a workgroup is already
+// running), publish the sum of their counts, and look back over their predecessors' status words, 64 at a
+// time, until they meet one that already knows its inclusive prefix.  `masks` (O2 <= 64 only, else null) keeps
+// each column's bin mask for the fill kernel; `total` (may be null) receives the number of output rows.
+#ifndef SPH_COUNT_BLOCKS
+#define SPH_COUNT_BLOCKS 256
+#endif
+constexpr int kCountPasses = 8; // most batches of 64 columns per workgroup (one wave scans each: kCountPasses <= waves)
+static_assert(kCountPasses <= kCountThreads / kWave, "a wave per batch");
+
 __global__ __launch_bounds__(kCountThreads) void outcoords_count_kernel(OutArgs a, int32_t *oz_ptr,
                                                                         unsigned long long *masks, int *state,
-                                                                        int32_t *total)
+                                                                        int32_t *total, int passes)
 {
-    __shared__ int s_ticket, s_last;
-    __shared__ int s_cnt[kCountCols];
+    __shared__ int s_ticket, s_excl;
+    __shared__ int s_cnt[kCountPasses][kCountCols];
+    __shared__ int s_tot[kCountPasses];
     const int ncol = a.B * a.O.n0 * a.O.n1;
-    const int nblocks = count_blocks(ncol);
+    const int nblocks = gridDim.x;
     unsigned long long *status = (unsigned long long *)(state + 2);
     const int tid = threadIdx.x;
-    if (tid == 0) {
-        s_ticket = atomicAdd(&state[0], 1);
-        s_last = 0;
-    }
+    if (tid == 0) s_ticket = atomicAdd(&state[0], 1);
     __syncthreads();
     const int t = s_ticket;
     const int part = tid % kColLanes, cl = tid / kColLanes;
-    const int oc = t * kCountCols + cl;
-    int cnt = 0;
-    if (oc < ncol) { // whole 16-lane groups take this branch together
-        const int nchunk = (a.O.n2 + 63) >> 6;
-        const int b = oc / (a.O.n0 * a.O.n1);
-        const int rem = oc - b * (a.O.n0 * a.O.n1);
-        const int o0 = rem / a.O.n1, o1 = rem % a.O.n1;
-        for (int ch = 0; ch < nchunk; ch++) {
-            const unsigned long long m = or_reduce16(column_mask(a, b, o0, o1, ch, part, kColLanes));
-            cnt += __popcll(m);
-            if (masks && part == 0) masks[oc] = m;
+    const int lane = tid & (kWave - 1), wave = tid / kWave;
+    const int col0 = t * passes * kCountCols; // first column of this workgroup
+    for (int p = 0; p < passes; p++) {
+        const int oc = col0 + p * kCountCols + cl;
+        int cnt = 0;
+        if (oc < ncol) { // whole 16-lane groups take this branch together
+            const int nchunk = (a.O.n2 + 63) >> 6;
+            const int b = oc / (a.O.n0 * a.O.n1);
+            const int rem = oc - b * (a.O.n0 * a.O.n1);
+            const int o0 = rem / a.O.n1, o1 = rem % a.O.n1;
+            for (int ch = 0; ch < nchunk; ch++) {
+                const unsigned long long m = or_reduce16(column_mask(a, b, o0, o1, ch, part, kColLanes));
+                cnt += __popcll(m);
+                if (masks && part == 0) masks[oc] = m;
+            }
         }
+        if (part == 0) s_cnt[p][cl] = cnt;
     }
-    if (part == 0) s_cnt[cl] = cnt;
     __syncthreads();
-    if (tid < kWave) {
-        const int lane = tid;
-        int incl = s_cnt[lane];
+    // wave p scans batch p
+    int incl = 0;
+    if (wave < passes) {
+        incl = lane < kCountCols ? s_cnt[wave][lane] : 0;
 #pragma unroll
-        for (int off = 1; off < kWave; off <<= 1) {
+        for (int off = 1; off < kCountCols; off <<= 1) {
             const int v = __shfl_up(incl, off, kWave);
             if (lane >= off) incl += v;
         }
-        const int agg = __shfl(incl, kWave - 1, kWave);
+        if (lane == kCountCols - 1) s_tot[wave] = incl;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        int agg = 0;
+        for (int p = 0; p < passes; p++) agg += s_tot[p];
         int excl = 0;
         if (t > 0) {
             if (lane == 0) status_store(&status[t], kScanAggregate | (unsigned)agg);
@@ -691,22 +713,18 @@ __global__ __launch_bounds__(kCountThreads) void outcoords_count_kernel(OutArgs 
                 base -= kWave;
             }
         }
-        if (lane == 0) status_store(&status[t], kScanInclusive | (unsigned)(excl + agg));
-        const int c = t * kCountCols + lane;
-        if (c < ncol) oz_ptr[c] = excl + incl;
         if (lane == 0) {
+            status_store(&status[t], kScanInclusive | (unsigned)(excl + agg));
+            s_excl = excl;
             if (t == nblocks - 1 && total) *total = excl + agg;
-            // this workgroup reads no status word any more
-            if (atomicAdd(&state[1], 1) == nblocks - 1) s_last = 1;
         }
     }
     __syncthreads();
-    if (s_last) { // every workgroup has finished its look-back: leave the state as it was found
-        for (int i = tid; i < nblocks; i += kCountThreads) status_store(&status[i], 0ull);
-        if (tid == 0) {
-            __hip_atomic_store(&state[0], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&state[1], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+    if (wave < passes) {
+        int before = s_excl;
+        for (int p = 0; p < wave; p++) before += s_tot[p];
+        const int c = col0 + wave * kCountCols + lane;
+        if (lane < kCountCols && c < ncol) oz_ptr[c] = before + incl;
     }
 }
 
@@ -989,8 +1007,20 @@ static int outcoords_count(const char *who, const int32_t *z_idx, const int32_t 
     SPH_REQUIRE(z_ptr && oz_ptr && scratch && in_rows >= 0 && (in_rows == 0 || z_idx), SPH_ERR_ARG, "%s: null argument", who);
     SPH_REQUIRE((uintptr_t)scratch % 8 == 0, SPH_ERR_ARG, "%s: scratch must be 8-byte aligned", who);
     const long ncol = (long)g->B * g->O[0] * g->O[1];
-    hipLaunchKernelGGL(outcoords_count_kernel, dim3(count_blocks(ncol)), dim3(kCountThreads), 0, (hipStream_t)stream,
-                       out_args(z_idx, z_ptr, in_rows, g), oz_ptr, outcoords_masks(g, scratch), (int *)scratch, total);
+    // batches of 64 columns per workgroup: as many as leave about 256 workgroups, one for small grids, which
+    // need every workgroup they can get to fill the chip.  Every workgroup costs an atomic on the one ticket
+    // counter, and those queue up at about 20 ns each (configuration 3, 131 072 columns: 74 us with 2048
+    // workgroups, 39 with 512, 32 with 256; whether one wave or the whole workgroup looks back makes no difference)
+    int passes = (int)(count_blocks(ncol) / SPH_COUNT_BLOCKS);
+    passes = passes < 1 ? 1 : (passes > kCountPasses ? kCountPasses : passes);
+    const int nblocks = (count_blocks(ncol) + passes - 1) / passes;
+    // the state of the scan starts at zero
+    const long nstate = 2 + 2 * (long)nblocks;
+    hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((nstate + 255) / 256)), dim3(256), 0, (hipStream_t)stream, scratch,
+                       nstate, 0);
+    hipLaunchKernelGGL(outcoords_count_kernel, dim3(nblocks), dim3(kCountThreads), 0, (hipStream_t)stream,
+                       out_args(z_idx, z_ptr, in_rows, g), oz_ptr, outcoords_masks(g, scratch), (int *)scratch, total,
+                       passes);
     return sph_check_launch(who);
 }
 
@@ -1047,11 +1077,6 @@ SPH_EXPORT int sph_outcoords_count_static(const int32_t *z_idx, const int32_t *z
                 "with a scratch of the caller's", who, ncol, kStaticCols);
     int32_t *ptr = nullptr;
     int rc = static_scratch_ptr(who, &ptr);
-    if (rc) return rc;
-    // the scan's state must start at zero; a launch leaves it so, but one that was cut short would not
-    const long n = scan_state_ints(ncol);
-    hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, ptr, n, 0);
-    rc = sph_check_launch(who);
     if (rc) return rc;
     rc = outcoords_count(who, z_idx, z_ptr, in_rows, g, oz_ptr, ptr, total_dev, stream);
     if (rc == SPH_OK && scratch_out) *scratch_out = ptr;

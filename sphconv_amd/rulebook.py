@@ -228,7 +228,7 @@ class RuleBook:
                                             L.ptr(scratch), total.data_ptr(), stream.cuda_stream))
             stream.synchronize()             # the one wait of a strided layer (the reference's is rules.cu:461)
         except Exception:
-            _WORKSPACES.pop(_workspace_key(dev), None)   # the scan's state may not be zero any more
+            _WORKSPACES.pop(_workspace_key(dev), None)   # whatever failed, the next call starts from fresh buffers
             raise
         out_rows = int(total[0])
         oz_idx = torch.empty(out_rows, dtype=torch.int32, device=dev)
@@ -337,9 +337,8 @@ class RuleBook:
         return [-(-self.out_shape[0] // int(tile_size[0])), -(-self.out_shape[1] // int(tile_size[1]))]
 
 
-# Scratch of the output-coordinate kernels, kept per (device, stream): the head of it is the state of the
-# scan across workgroups, which must be zero when a count is enqueued and is left zero by it, so it is
-# zeroed once, when it is allocated.  With it, one pinned host int that receives the output row count.
+# Scratch of the output-coordinate kernels, kept per (device, stream), and one pinned host int that receives
+# the output row count.
 _WORKSPACES = {}
 
 
@@ -353,7 +352,7 @@ def _outcoords_workspace(dev, nints: int):
     key = _workspace_key(dev)
     ws = _WORKSPACES.get(key)
     if ws is None or ws[0].numel() < nints:
-        scratch = torch.zeros(max(nints + (nints & 1), 1 << 16), dtype=torch.int32, device=dev)
+        scratch = torch.empty(max(nints + (nints & 1), 1 << 16), dtype=torch.int32, device=dev)
         total = ws[1] if ws is not None else torch.zeros(1, dtype=torch.int32).pin_memory()
         ws = (scratch, total)
         _WORKSPACES[key] = ws

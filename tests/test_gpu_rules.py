@@ -262,8 +262,8 @@ def test_unsorted_long_fibers_take_the_general_join():
 
 def test_outcoords_total_is_optional():
     """sph_outcoords_count writes the output row count to *total_dev when given one; either way the count is
-    the last element of the scanned oz_ptr.  The head of the scratch (the state of the scan across workgroups)
-    must be zero on entry and is zero again afterwards, so one zeroed scratch serves call after call."""
+    the last element of the scanned oz_ptr.  The scratch may hold anything on entry (the call clears the state
+    of the scan across workgroups itself), so one scratch serves call after call."""
     import ctypes as C
     from sphconv_amd import _lib as L
     rng = np.random.default_rng(5)
@@ -277,7 +277,7 @@ def test_outcoords_total_is_optional():
     ns = lib.sph_outcoords_state_ints(C.byref(g))
     assert 0 < ns <= n
     ptrs = []
-    scratch = torch.zeros(n + (n & 1), dtype=torch.int32, device="cuda:0")
+    scratch = torch.full((n + (n & 1),), -1, dtype=torch.int32, device="cuda:0")    # garbage on entry
     for with_total in (True, False):
         oz_ptr = torch.empty((B, out_shape[0], out_shape[1]), dtype=torch.int32, device="cuda:0")
         total = torch.full((1,), -7, dtype=torch.int32, device="cuda:0")
@@ -285,17 +285,18 @@ def test_outcoords_total_is_optional():
                                         L.ptr(scratch), L.ptr(total) if with_total else None, L.stream()))
         torch.cuda.synchronize()
         assert int(total.item()) == (int(oz_ptr.view(-1)[-1].item()) if with_total else -7)
-        assert int(scratch[:ns].abs().sum().item()) == 0
         ptrs.append(oz_ptr.cpu().numpy())
     assert np.array_equal(ptrs[0], ptrs[1])
     book = RuleBook.build(zi, zp, B, shape, out_shape, [3, 3, 3], [2, 2, 2], [1, 1, 1])
     assert np.array_equal(book.oz_ptr.cpu().numpy(), ptrs[0]) and book.out_rows == int(ptrs[0].reshape(-1)[-1])
 
 
-@pytest.mark.parametrize("shape,p", [([40, 700, 20], 0.02), ([64, 1024, 70], 0.05), ([3, 21, 9], 0.5)])
+@pytest.mark.parametrize("shape,p", [([40, 700, 20], 0.02), ([64, 1024, 70], 0.05), ([3, 21, 9], 0.5),
+                                     ([500, 599, 8], 0.01)])
 def test_outcoords_scan_over_many_workgroups(shape, p):
-    """The scan of the per-column counts runs inside the count kernel, across its workgroups of 64 columns:
-    grids of one workgroup, of hundreds (look-back over several windows of 64 predecessors) and with more
+    """The scan of the per-column counts runs inside the count kernel, across its workgroups of 64 to 512
+    columns: grids of one workgroup, of hundreds (look-back over several windows of 64 predecessors), with
+    one, three and eight batches of 64 columns per workgroup (the last grid ends inside a batch) and with more
     than 64 bins (no masks kept), twice in a row on the same scratch, against numpy's cumsum."""
     import ctypes as C
     from sphconv_amd import _lib as L
@@ -311,7 +312,7 @@ def test_outcoords_scan_over_many_workgroups(shape, p):
     lib = L.lib()
     g = L.make_geom(B, shape, out_shape, [3, 3, 3], [2, 2, 2], [1, 1, 1], [1, 1, 1])
     n = lib.sph_outcoords_scratch_ints(C.byref(g))
-    scratch = torch.zeros(n + (n & 1), dtype=torch.int32, device="cuda:0")
+    scratch = torch.empty(n + (n & 1), dtype=torch.int32, device="cuda:0")
     zi, zp = G.t(z_idx), G.t(z_ptr)
     for _ in range(2):
         oz_ptr = torch.full((B, out_shape[0], out_shape[1]), -1, dtype=torch.int32, device="cuda:0")
