@@ -139,7 +139,8 @@ int sph_rules_build_pack(const int32_t *z_idx, const int32_t *z_ptr, int in_rows
  *     `scratch`: 8-byte aligned device memory of sph_outcoords_scratch_ints(g) int32, contents arbitrary;
  *     its first sph_outcoords_state_ints(g) entries hold the state of the scan across workgroups, which a
  *     small fill kernel in front of the count kernel clears (calls that overlap on one scratch race).
- *     Behind the state, when O[2] <= 64, each column's 64-bit mask of active bins is kept for step 2.
+ *     Behind the state, when O[2] <= 512, each column's 64-bit masks of active bins (one per 64 bins) are
+ *     kept for step 2; deeper grids keep none and step 2 walks the fibers again.
  *  2. once the caller knows the total: sph_outcoords_fill, given the same scratch and oz_ptr, writes
  *     oz_idx (ascending within a column).
  * sph_outcoords_blocks(g) = ceil(columns / 256), the grid of the fill kernel. */
@@ -158,7 +159,8 @@ int sph_outcoords_fill(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
  * kernels and results as sph_outcoords_count, but the scratch is an array of the library's own
  * (8.1 MiB of static device memory on each GPU the library runs on, held until the process ends),
  * so the call allocates and frees nothing.  It serves grids of up to SPH_STATIC_MAX_COLUMNS output
- * columns (B * O[0] * O[1]) and refuses larger ones with SPH_ERR_UNSUPPORTED.  *scratch_out (may be
+ * columns (B * O[0] * O[1]; with 64 < O[2] <= 512 a column counts ceil(O[2] / 64) times, once per mask
+ * it keeps) and refuses larger ones with SPH_ERR_UNSUPPORTED.  *scratch_out (may be
  * null) receives the array's device address on the current GPU: pass it as `scratch` to
  * sph_outcoords_fill.  Every call on a GPU shares that GPU's array, which keeps the last call's
  * contents (the call clears the part that must start at zero): calls that overlap on one GPU race,

@@ -588,6 +588,56 @@ __device__ unsigned long long column_mask(const OutArgs &a, int b, int o0, int o
     return mask;
 }
 
+// The same walk for the first NCH chunks of 64 bins at once (O2 <= 64 * NCH): the fibers are read once, not once
+// per chunk.  The chunk of a bin is matched against constants, so the masks stay in registers.
+template <int NCH>
+__device__ __forceinline__ void column_masks(const OutArgs &a, int b, int o0, int o1, int part, int step,
+                                             unsigned long long (&mask)[NCH])
+{
+#pragma unroll
+    for (int c = 0; c < NCH; c++) mask[c] = 0;
+    const int K01 = a.cv.K0 * a.cv.K1;
+    const bool pow2 = (a.cv.s2 & (a.cv.s2 - 1)) == 0;
+    const int sh2 = __ffs(a.cv.s2) - 1;
+    for (int k01 = part; k01 < K01; k01 += step) {
+        const int k0 = k01 / a.cv.K1, k1 = k01 - k0 * a.cv.K1;
+        int x0 = o0 * a.cv.s0 - a.cv.p0 + k0;
+        int x1 = o1 * a.cv.s1 - a.cv.p1 + k1;
+        if (x0 < 0 || x0 >= a.S.n0 || x1 < 0 || x1 >= a.S.n1) continue;
+        int pc = (b * a.S.n0 + x0) * a.S.n1 + x1;
+        int ps, pe;
+        fiber_range(a.z_ptr, pc, a.in_rows, ps, pe);
+        for (int e0 = ps; e0 < pe; e0 += 4) {
+            int z[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) z[q] = a.z_idx[min(e0 + q, pe - 1)];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                if (e0 + q >= pe) continue;
+                for (int k2 = 0; k2 < a.cv.K2; k2++) {
+                    int t = z[q] + a.cv.p2 - k2;
+                    int o2;
+                    if (pow2) {
+                        if (t < 0 || (t & (a.cv.s2 - 1))) continue;
+                        o2 = t >> sh2;
+                    } else {
+                        if (t < 0 || t % a.cv.s2) continue;
+                        o2 = t / a.cv.s2;
+                    }
+                    if (o2 >= a.O.n2) continue;
+                    const unsigned long long bit = 1ull << (o2 & 63);
+                    const int ch = o2 >> 6;
+#pragma unroll
+                    for (int c = 0; c < NCH; c++) mask[c] |= ch == c ? bit : 0ull;
+                }
+            }
+        }
+    }
+}
+
+constexpr int kMaskChunks = 8;                   // chunks of 64 bins (O2 <= 512) up to which every column's masks are kept
+__host__ __device__ inline int mask_chunks(int O2) { return (O2 + 63) >> 6; }
+
 constexpr int kColLanes = 16;                    // lanes that share one output column
 #ifndef SPH_COUNT_COLS
 #define SPH_COUNT_COLS 64
@@ -606,6 +656,24 @@ __device__ __forceinline__ unsigned long long or_reduce16(unsigned long long m)
         hi |= __shfl_xor(hi, off, kWave);
     }
     return ((unsigned long long)hi << 32) | lo;
+}
+
+// Active bins of one output column, counted by its 16 lanes in one walk over the fibers that reach it; the
+// masks of its nchunk <= NCH chunks go to masks[oc * nchunk + chunk] (masks may be null).
+template <int NCH>
+__device__ __forceinline__ int count_column(const OutArgs &a, int b, int o0, int o1, int part, unsigned long long *masks,
+                                            int oc, int nchunk)
+{
+    unsigned long long m[NCH];
+    column_masks<NCH>(a, b, o0, o1, part, kColLanes, m);
+    int cnt = 0;
+#pragma unroll
+    for (int c = 0; c < NCH; c++) {
+        m[c] = or_reduce16(m[c]);
+        cnt += __popcll(m[c]);
+        if (masks && part == 0 && c < nchunk) masks[(long)oc * nchunk + c] = m[c];
+    }
+    return cnt;
 }
 
 // State of the scan across workgroups, at the head of the caller's scratch: a ticket counter (and a spare
@@ -663,14 +731,21 @@ __global__ __launch_bounds__(kCountThreads) void outcoords_count_kernel(OutArgs 
         const int oc = col0 + p * kCountCols + cl;
         int cnt = 0;
         if (oc < ncol) { // whole 16-lane groups take this branch together
-            const int nchunk = (a.O.n2 + 63) >> 6;
+            const int nchunk = mask_chunks(a.O.n2);
             const int b = oc / (a.O.n0 * a.O.n1);
             const int rem = oc - b * (a.O.n0 * a.O.n1);
             const int o0 = rem / a.O.n1, o1 = rem % a.O.n1;
-            for (int ch = 0; ch < nchunk; ch++) {
-                const unsigned long long m = or_reduce16(column_mask(a, b, o0, o1, ch, part, kColLanes));
-                cnt += __popcll(m);
-                if (masks && part == 0) masks[oc] = m;
+            if (nchunk == 1) {
+                cnt = count_column<1>(a, b, o0, o1, part, masks, oc, nchunk);
+            } else if (nchunk <= 2) {
+                cnt = count_column<2>(a, b, o0, o1, part, masks, oc, nchunk);
+            } else if (nchunk <= 4) {
+                cnt = count_column<4>(a, b, o0, o1, part, masks, oc, nchunk);
+            } else if (nchunk <= kMaskChunks) {
+                cnt = count_column<kMaskChunks>(a, b, o0, o1, part, masks, oc, nchunk);
+            } else { // deeper grids: one walk per chunk, nothing kept
+                for (int ch = 0; ch < nchunk; ch++)
+                    cnt += __popcll(or_reduce16(column_mask(a, b, o0, o1, ch, part, kColLanes)));
             }
         }
         if (part == 0) s_cnt[p][cl] = cnt;
@@ -743,7 +818,7 @@ __global__ __launch_bounds__(kThreads) void outcoords_fill_kernel(OutArgs a, con
     int o0 = rem / a.O.n1, o1 = rem % a.O.n1;
     int nchunk = (a.O.n2 + 63) >> 6;
     for (int ch = 0; ch < nchunk; ch++) {
-        unsigned long long m = masks ? masks[oc] : column_mask(a, b, o0, o1, ch, 0, 1);
+        unsigned long long m = masks ? masks[(long)oc * nchunk + ch] : column_mask(a, b, o0, o1, ch, 0, 1);
         while (m) {
             int bit = __ffsll((long long)m) - 1;
             if (pos < out_rows) oz_idx[pos] = ch * 64 + bit;
@@ -979,14 +1054,15 @@ SPH_EXPORT int sph_outcoords_scratch_ints(const sph_geom *g)
 {
     SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_scratch_ints: bad geometry");
     const long ncol = (long)g->B * g->O[0] * g->O[1];
-    const long n = scan_state_ints(ncol) + (g->O[2] <= 64 ? 2 * ncol : 0);
+    const int nchunk = mask_chunks(g->O[2]);
+    const long n = scan_state_ints(ncol) + (nchunk <= kMaskChunks ? 2 * ncol * nchunk : 0);
     SPH_REQUIRE(n < 2147483647L, SPH_ERR_UNSUPPORTED, "sph_outcoords_scratch_ints: grid too large");
     return (int)n;
 }
 
 static unsigned long long *outcoords_masks(const sph_geom *g, int32_t *scratch)
 {
-    if (g->O[2] > 64) return nullptr;
+    if (mask_chunks(g->O[2]) > kMaskChunks) return nullptr;
     return (unsigned long long *)(scratch + scan_state_ints((long)g->B * g->O[0] * g->O[1]));
 }
 
@@ -1072,9 +1148,12 @@ SPH_EXPORT int sph_outcoords_count_static(const int32_t *z_idx, const int32_t *z
     const char *who = "sph_outcoords_count_static";
     SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "%s: bad geometry", who);
     const long ncol = (long)g->B * g->O[0] * g->O[1];
-    SPH_REQUIRE(ncol <= kStaticCols, SPH_ERR_UNSUPPORTED,
-                "%s: %ld output columns (B*O0*O1), the library's own scratch provides for %ld: use sph_outcoords_count "
-                "with a scratch of the caller's", who, ncol, kStaticCols);
+    // a column keeps one 64-bit mask per 64 bins of O2 (up to 512 bins; deeper grids keep none)
+    const int nchunk = mask_chunks(g->O[2]);
+    const long need = ncol * (nchunk <= kMaskChunks ? nchunk : 1);
+    SPH_REQUIRE(need <= kStaticCols, SPH_ERR_UNSUPPORTED,
+                "%s: %ld output columns (B*O0*O1) of %d bins need %ld mask words, the library's own scratch provides for "
+                "%ld: use sph_outcoords_count with a scratch of the caller's", who, ncol, g->O[2], need, kStaticCols);
     int32_t *ptr = nullptr;
     int rc = static_scratch_ptr(who, &ptr);
     if (rc) return rc;

@@ -292,12 +292,14 @@ def test_outcoords_total_is_optional():
 
 
 @pytest.mark.parametrize("shape,p", [([40, 700, 20], 0.02), ([64, 1024, 70], 0.05), ([3, 21, 9], 0.5),
-                                     ([500, 599, 8], 0.01)])
+                                     ([500, 599, 8], 0.01), ([10, 30, 400], 0.05), ([12, 20, 250], 0.05),
+                                     ([6, 20, 1100], 0.02)])
 def test_outcoords_scan_over_many_workgroups(shape, p):
     """The scan of the per-column counts runs inside the count kernel, across its workgroups of 64 to 512
     columns: grids of one workgroup, of hundreds (look-back over several windows of 64 predecessors), with
-    one, three and eight batches of 64 columns per workgroup (the last grid ends inside a batch) and with more
-    than 64 bins (no masks kept), twice in a row on the same scratch, against numpy's cumsum."""
+    one, three and eight batches of 64 columns per workgroup (one grid ends inside a batch), and output
+    columns of 125, 200 and 550 bins (two and four masks per column kept; none beyond 512 bins), twice in a row on
+    the same scratch, against numpy's cumsum and the active set of a dense convolution."""
     import ctypes as C
     from sphconv_amd import _lib as L
     rng = np.random.default_rng(shape[1])
@@ -322,3 +324,9 @@ def test_outcoords_scan_over_many_workgroups(shape, p):
         torch.cuda.current_stream().synchronize()
         assert int(total[0]) == int(want[-1])            # written by the kernel to pinned host memory
         assert np.array_equal(oz_ptr.cpu().numpy().reshape(-1), want)
+        # the bins themselves: from the masks the count kernel kept (up to 512 bins) or from a second walk
+        m = int(total[0])
+        oz_idx = torch.full((max(m, 1),), -1, dtype=torch.int32, device="cuda:0")
+        L.check(lib.sph_outcoords_fill(L.ptr(zi), L.ptr(zp), int(zi.shape[0]), C.byref(g), L.ptr(scratch),
+                                       L.ptr(oz_ptr), L.ptr(oz_idx), m, L.stream()))
+        assert np.array_equal(oz_idx.cpu().numpy()[:m], np.nonzero(act.numpy())[3].astype(np.int32))

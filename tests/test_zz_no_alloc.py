@@ -50,7 +50,8 @@ def _run(lib, zi, zp, B, shape, out_shape, static):
 def test_static_scratch_matches_caller_scratch_twice():
     lib = L.lib()
     # first a grid of hundreds of scan workgroups, then a much smaller one: the array keeps the first call's contents
-    for seed, B, shape, p in ((1, 4, [64, 512, 32], 0.05), (2, 1, [9, 33, 12], 0.3)):
+    # (and last one whose columns keep three masks each: 150 bins)
+    for seed, B, shape, p in ((1, 4, [64, 512, 32], 0.05), (2, 1, [9, 33, 12], 0.3), (3, 2, [16, 40, 300], 0.05)):
         zi, zp, out_shape = _case(seed, B, shape, p)
         got = _run(lib, zi, zp, B, shape, out_shape, static=True)
         want = _run(lib, zi, zp, B, shape, out_shape, static=False)
