@@ -131,14 +131,14 @@ int sph_rules_build_pack(const int32_t *z_idx, const int32_t *z_ptr, int in_rows
 
 /* Replaces the output-coordinate half of get_rules (rules.cu:417-443, 461-462: prepareGridKernel, two
  * cumsums, roll/index_put/add and the device->host read), in two steps because the caller must size oz_idx:
- *  1. sph_outcoords_count: one kernel counts every output column's active bins and scans the counts
- *     (single pass: workgroups of 64 to 512 columns look back over their predecessors' sums) into oz_ptr
- *     (inclusive), and writes the number of output rows to *total_dev (null: not written; it is also the
+ *  1. sph_outcoords_count: counts every output column's active bins into oz_ptr and scans them in place
+ *     (inclusive; one pass over the counts: tiles of 2048 columns look back over their predecessors'
+ *     sums), and writes the number of output rows to *total_dev (null: not written; it is also the
  *     last element of oz_ptr).  total_dev is any address the GPU can write: device memory, or pinned host
  *     memory (hipHostMalloc) that the host reads after synchronising the stream, without a copy.
  *     `scratch`: 8-byte aligned device memory of sph_outcoords_scratch_ints(g) int32, contents arbitrary;
  *     its first sph_outcoords_state_ints(g) entries hold the state of the scan across workgroups, which a
- *     small fill kernel in front of the count kernel clears (calls that overlap on one scratch race).
+ *     small fill kernel in front of the scan clears (calls that overlap on one scratch race).
  *     Behind the state, when O[2] <= 512, each column's 64-bit masks of active bins (one per 64 bins) are
  *     kept for step 2; deeper grids keep none and step 2 walks the fibers again.
  *  2. once the caller knows the total: sph_outcoords_fill, given the same scratch and oz_ptr, writes
@@ -157,7 +157,7 @@ int sph_outcoords_fill(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
 /* sph_outcoords_count for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
  * kernels and results as sph_outcoords_count, but the scratch is an array of the library's own
- * (8.1 MiB of static device memory on each GPU the library runs on, held until the process ends),
+ * (8.0 MiB of static device memory on each GPU the library runs on, held until the process ends),
  * so the call allocates and frees nothing.  It serves grids of up to SPH_STATIC_MAX_COLUMNS output
  * columns (B * O[0] * O[1]; with 64 < O[2] <= 512 a column counts ceil(O[2] / 64) times, once per mask
  * it keeps) and refuses larger ones with SPH_ERR_UNSUPPORTED.  *scratch_out (may be

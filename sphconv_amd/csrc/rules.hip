@@ -7,6 +7,7 @@
 // All kernels are integer and HBM/latency bound.
 #include "common.h"
 #include "pack.h"
+#include "scan.h"
 
 #include <cstring>
 #include <mutex>
@@ -639,11 +640,7 @@ constexpr int kMaskChunks = 8;                   // chunks of 64 bins (O2 <= 512
 __host__ __device__ inline int mask_chunks(int O2) { return (O2 + 63) >> 6; }
 
 constexpr int kColLanes = 16;                    // lanes that share one output column
-#ifndef SPH_COUNT_COLS
-#define SPH_COUNT_COLS 64
-#endif
-constexpr int kCountCols = SPH_COUNT_COLS;       // output columns per workgroup of the count kernel (at most 64)
-static_assert(kCountCols <= kWave && (kCountCols & (kCountCols - 1)) == 0, "one wave scans a workgroup's counts");
+constexpr int kCountCols = 16;                   // output columns per workgroup of the count kernel
 constexpr int kCountThreads = kCountCols * kColLanes;
 
 // OR over the 16 lanes of a column group (all 16 are active together).
@@ -676,131 +673,43 @@ __device__ __forceinline__ int count_column(const OutArgs &a, int b, int o0, int
     return cnt;
 }
 
-// State of the scan across workgroups, at the head of the caller's scratch: a ticket counter (and a spare
-// word that keeps the status words 8-byte aligned) and one 64-bit status word per workgroup (flag in the two
-// top bits, value in the low 32).  A fill kernel clears it in front of every count launch: a counter of
-// finished workgroups, by which the last one could clear it instead, costs every workgroup a second atomic on
-// one address, and those queue up behind one another across the XCDs.
-constexpr unsigned long long kScanAggregate = 1ull << 62; // value = sum of the workgroup's own counts
-constexpr unsigned long long kScanInclusive = 2ull << 62; // value = sum of all counts up to and including it
-__host__ __device__ inline int count_blocks(long ncol) { return (int)((ncol + kCountCols - 1) / kCountCols); }
-__host__ __device__ inline long scan_state_ints(long ncol) { return 2 + 2 * (long)count_blocks(ncol); }
+// Scratch of the output-coordinate kernels: the state of the scan of the counts (sph_scan, one 64-bit word per
+// tile of 2048 columns) at its head, the columns' bin masks behind it.
+inline long scan_state_ints(long ncol) { return (long)(sph_scan::state_bytes(ncol) / 4); }
 
-__device__ __forceinline__ unsigned long long status_load(const unsigned long long *p)
+// Per-column counts.  16 lanes share an output column (one input column (k0, k1) each, K0*K1 = 9 of them busy
+// for a 3x3x3 kernel), so the fibers that reach a column are walked side by side and small grids still fill
+// the chip.  The counts go to oz_ptr, which sph_scan then scans in place: a scan folded into this kernel
+// (workgroups numbered by a ticket, decoupled look-back) was measured slower than the two kernels, because
+// every workgroup then pays an atomic on the one ticket counter and same-address device-scope atomics queue
+// at about 20 ns each, while the counting wants thousands of small workgroups (131 072 columns: 74 us with
+// 2048 workgroups of 64 columns, 31 us with 256 of 512 columns, against 19 us here + 6 us of scan).
+// `masks` (O2 <= 512 only, else null) keeps each column's bin masks for the fill kernel.
+__global__ __launch_bounds__(kCountThreads) void outcoords_count_kernel(OutArgs a, int32_t *counts,
+                                                                        unsigned long long *masks)
 {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void status_store(unsigned long long *p, unsigned long long v)
-{
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Per-column counts and their inclusive scan (oz_ptr) in one launch.  16 lanes share an output column (one
-// input column (k0, k1) each, K0*K1 = 9 of them busy for a 3x3x3 kernel), so the fibers that reach a column
-// are walked side by side and small grids still fill the chip; a workgroup takes `passes` batches of 64
-// consecutive columns (the launcher gives large grids several, so that a few hundred workgroups share the
-// ticket counter and the status words: with one batch each, 2048 workgroups spent most of the kernel queueing
-// for them).  Workgroups number themselves by a ticket (so every predecessor of a workgroup is already
-// running), publish the sum of their counts, and look back over their predecessors' status words, 64 at a
-// time, until they meet one that already knows its inclusive prefix.  `masks` (O2 <= 64 only, else null) keeps
-// each column's bin mask for the fill kernel; `total` (may be null) receives the number of output rows.
-#ifndef SPH_COUNT_BLOCKS
-#define SPH_COUNT_BLOCKS 256
-#endif
-constexpr int kCountPasses = 8; // most batches of 64 columns per workgroup (one wave scans each: kCountPasses <= waves)
-static_assert(kCountPasses <= kCountThreads / kWave, "a wave per batch");
-
-__global__ __launch_bounds__(kCountThreads) void outcoords_count_kernel(OutArgs a, int32_t *oz_ptr,
-                                                                        unsigned long long *masks, int *state,
-                                                                        int32_t *total, int passes)
-{
-    __shared__ int s_ticket, s_excl;
-    __shared__ int s_cnt[kCountPasses][kCountCols];
-    __shared__ int s_tot[kCountPasses];
     const int ncol = a.B * a.O.n0 * a.O.n1;
-    const int nblocks = gridDim.x;
-    unsigned long long *status = (unsigned long long *)(state + 2);
     const int tid = threadIdx.x;
-    if (tid == 0) s_ticket = atomicAdd(&state[0], 1);
-    __syncthreads();
-    const int t = s_ticket;
     const int part = tid % kColLanes, cl = tid / kColLanes;
-    const int lane = tid & (kWave - 1), wave = tid / kWave;
-    const int col0 = t * passes * kCountCols; // first column of this workgroup
-    for (int p = 0; p < passes; p++) {
-        const int oc = col0 + p * kCountCols + cl;
-        int cnt = 0;
-        if (oc < ncol) { // whole 16-lane groups take this branch together
-            const int nchunk = mask_chunks(a.O.n2);
-            const int b = oc / (a.O.n0 * a.O.n1);
-            const int rem = oc - b * (a.O.n0 * a.O.n1);
-            const int o0 = rem / a.O.n1, o1 = rem % a.O.n1;
-            if (nchunk == 1) {
-                cnt = count_column<1>(a, b, o0, o1, part, masks, oc, nchunk);
-            } else if (nchunk <= 2) {
-                cnt = count_column<2>(a, b, o0, o1, part, masks, oc, nchunk);
-            } else if (nchunk <= 4) {
-                cnt = count_column<4>(a, b, o0, o1, part, masks, oc, nchunk);
-            } else if (nchunk <= kMaskChunks) {
-                cnt = count_column<kMaskChunks>(a, b, o0, o1, part, masks, oc, nchunk);
-            } else { // deeper grids: one walk per chunk, nothing kept
-                for (int ch = 0; ch < nchunk; ch++)
-                    cnt += __popcll(or_reduce16(column_mask(a, b, o0, o1, ch, part, kColLanes)));
-            }
-        }
-        if (part == 0) s_cnt[p][cl] = cnt;
+    const int oc = blockIdx.x * kCountCols + cl;
+    if (oc >= ncol) return; // whole 16-lane groups leave together
+    const int nchunk = mask_chunks(a.O.n2);
+    const int b = oc / (a.O.n0 * a.O.n1);
+    const int rem = oc - b * (a.O.n0 * a.O.n1);
+    const int o0 = rem / a.O.n1, o1 = rem % a.O.n1;
+    int cnt = 0;
+    if (nchunk == 1) {
+        cnt = count_column<1>(a, b, o0, o1, part, masks, oc, nchunk);
+    } else if (nchunk <= 2) {
+        cnt = count_column<2>(a, b, o0, o1, part, masks, oc, nchunk);
+    } else if (nchunk <= 4) {
+        cnt = count_column<4>(a, b, o0, o1, part, masks, oc, nchunk);
+    } else if (nchunk <= kMaskChunks) {
+        cnt = count_column<kMaskChunks>(a, b, o0, o1, part, masks, oc, nchunk);
+    } else { // deeper grids: one walk per chunk, nothing kept
+        for (int ch = 0; ch < nchunk; ch++) cnt += __popcll(or_reduce16(column_mask(a, b, o0, o1, ch, part, kColLanes)));
     }
-    __syncthreads();
-    // wave p scans batch p
-    int incl = 0;
-    if (wave < passes) {
-        incl = lane < kCountCols ? s_cnt[wave][lane] : 0;
-#pragma unroll
-        for (int off = 1; off < kCountCols; off <<= 1) {
-            const int v = __shfl_up(incl, off, kWave);
-            if (lane >= off) incl += v;
-        }
-        if (lane == kCountCols - 1) s_tot[wave] = incl;
-    }
-    __syncthreads();
-    if (wave == 0) {
-        int agg = 0;
-        for (int p = 0; p < passes; p++) agg += s_tot[p];
-        int excl = 0;
-        if (t > 0) {
-            if (lane == 0) status_store(&status[t], kScanAggregate | (unsigned)agg);
-            for (int base = t - 1;;) {
-                const int idx = base - lane; // lane 0 looks at the nearest predecessor
-                const unsigned long long w = idx >= 0 ? status_load(&status[idx]) : kScanInclusive; // before the first: 0
-                const unsigned long long flag = w >> 62;
-                const unsigned long long has_incl = __ballot(flag == 2), empty = __ballot(flag == 0);
-                const int fi = has_incl ? __ffsll((long long)has_incl) - 1 : kWave; // nearest inclusive prefix
-                const unsigned long long need = fi >= kWave - 1 ? ~0ull : (2ull << fi) - 1ull;
-                if (empty & need) { // a predecessor on the way has not published yet
-                    __builtin_amdgcn_s_sleep(1);
-                    continue;
-                }
-                int v = lane <= fi ? (int)(unsigned)w : 0;
-#pragma unroll
-                for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-                excl += v;
-                if (fi < kWave) break;
-                base -= kWave;
-            }
-        }
-        if (lane == 0) {
-            status_store(&status[t], kScanInclusive | (unsigned)(excl + agg));
-            s_excl = excl;
-            if (t == nblocks - 1 && total) *total = excl + agg;
-        }
-    }
-    __syncthreads();
-    if (wave < passes) {
-        int before = s_excl;
-        for (int p = 0; p < wave; p++) before += s_tot[p];
-        const int c = col0 + wave * kCountCols + lane;
-        if (lane < kCountCols && c < ncol) oz_ptr[c] = before + incl;
-    }
+    if (part == 0) counts[oc] = cnt;
 }
 
 // oz_ptr holds the inclusive scan of the counts; one thread writes the bins of one column.
@@ -1083,20 +992,17 @@ static int outcoords_count(const char *who, const int32_t *z_idx, const int32_t 
     SPH_REQUIRE(z_ptr && oz_ptr && scratch && in_rows >= 0 && (in_rows == 0 || z_idx), SPH_ERR_ARG, "%s: null argument", who);
     SPH_REQUIRE((uintptr_t)scratch % 8 == 0, SPH_ERR_ARG, "%s: scratch must be 8-byte aligned", who);
     const long ncol = (long)g->B * g->O[0] * g->O[1];
-    // batches of 64 columns per workgroup: as many as leave about 256 workgroups, one for small grids, which
-    // need every workgroup they can get to fill the chip.  Every workgroup costs an atomic on the one ticket
-    // counter, and those queue up at about 20 ns each (configuration 3, 131 072 columns: 74 us with 2048
-    // workgroups, 39 with 512, 32 with 256; whether one wave or the whole workgroup looks back makes no difference)
-    int passes = (int)(count_blocks(ncol) / SPH_COUNT_BLOCKS);
-    passes = passes < 1 ? 1 : (passes > kCountPasses ? kCountPasses : passes);
-    const int nblocks = (count_blocks(ncol) + passes - 1) / passes;
-    // the state of the scan starts at zero
-    const long nstate = 2 + 2 * (long)nblocks;
-    hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((nstate + 255) / 256)), dim3(256), 0, (hipStream_t)stream, scratch,
-                       nstate, 0);
+    const unsigned nblocks = (unsigned)((ncol + kCountCols - 1) / kCountCols);
     hipLaunchKernelGGL(outcoords_count_kernel, dim3(nblocks), dim3(kCountThreads), 0, (hipStream_t)stream,
-                       out_args(z_idx, z_ptr, in_rows, g), oz_ptr, outcoords_masks(g, scratch), (int *)scratch, total,
-                       passes);
+                       out_args(z_idx, z_ptr, in_rows, g), oz_ptr, outcoords_masks(g, scratch));
+    int rc = sph_check_launch(who);
+    if (rc) return rc;
+    // counts -> inclusive scan in place; the last tile also writes the row count
+    hipError_t e = sph_scan::launch<sph_scan::Plus, true>(oz_ptr, oz_ptr, ncol, scratch, 0, (hipStream_t)stream, total);
+    if (e != hipSuccess) {
+        sph_set_error("%s: scan: %s", who, hipGetErrorString(e));
+        return SPH_ERR_LAUNCH;
+    }
     return sph_check_launch(who);
 }
 
@@ -1112,8 +1018,8 @@ SPH_EXPORT int sph_outcoords_count(const int32_t *z_idx, const int32_t *z_ptr, i
 // Each GPU holds its own copy of the array at its own address, found once per device.
 // ---------------------------------------------------------------------------
 constexpr long kStaticCols = SPH_STATIC_MAX_COLUMNS; // output columns (B * O0 * O1) the library's own scratch provides for
-constexpr long kStaticInts = 2 + 2 * ((kStaticCols + kCountCols - 1) / kCountCols) + 2 * kStaticCols;
-static __device__ __align__(256) int32_t sph_static_scratch[kStaticInts]; // 8.1 MiB per GPU
+constexpr long kStaticInts = 256 + 2 * (kStaticCols / sph_scan::kTile) + 2 * kStaticCols; // scan state (rounded up) + masks
+static __device__ __align__(256) int32_t sph_static_scratch[kStaticInts]; // 8.0 MiB per GPU
 constexpr int kMaxDevices = 64;
 static int32_t *g_static_ptr[kMaxDevices];
 static std::mutex g_static_mutex;

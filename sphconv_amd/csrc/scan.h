@@ -41,8 +41,11 @@ static __global__ void clear_state_kernel(int *state, int nints)
 }
 
 // out[i] = op(in[0], ..., in[i]) (INCLUSIVE) or op(init, in[0], ..., in[i-1]) (exclusive; init counts first).
+// *total (may be null; any address the GPU can write, e.g. pinned host memory) receives op over all n elements
+// (and init, for an exclusive scan).
 template <class OP, bool INCLUSIVE>
-__global__ __launch_bounds__(kThreads) void scan_kernel(const int32_t *in, int32_t *out, long n, int *state, int init)
+__global__ __launch_bounds__(kThreads) void scan_kernel(const int32_t *in, int32_t *out, long n, int *state, int init,
+                                                        int32_t *total)
 {
     __shared__ int s_ticket;
     __shared__ int s_wave[kThreads / kWaveSize];
@@ -115,6 +118,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(const int32_t *in, int32
             __hip_atomic_store(&status[t], kInclusive | (unsigned)OP::op(excl, agg), __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
             s_prefix = excl;
+            if (total && t == (int)gridDim.x - 1) *total = OP::op(excl, agg);
         }
     }
     __syncthreads();
@@ -142,12 +146,14 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(const int32_t *in, int32
 
 // Enqueues the scan of n elements on st; state: state_bytes(n) bytes of device memory, 8-byte aligned.
 template <class OP, bool INCLUSIVE>
-inline hipError_t launch(const int32_t *in, int32_t *out, long n, void *state, int init, hipStream_t st)
+inline hipError_t launch(const int32_t *in, int32_t *out, long n, void *state, int init, hipStream_t st,
+                         int32_t *total = nullptr)
 {
     if (n <= 0) return hipSuccess;
     const int nt = tiles(n), nints = 2 + 2 * nt;
     hipLaunchKernelGGL(clear_state_kernel, dim3((nints + 255) / 256), dim3(256), 0, st, (int *)state, nints);
-    hipLaunchKernelGGL((scan_kernel<OP, INCLUSIVE>), dim3(nt), dim3(kThreads), 0, st, in, out, n, (int *)state, init);
+    hipLaunchKernelGGL((scan_kernel<OP, INCLUSIVE>), dim3(nt), dim3(kThreads), 0, st, in, out, n, (int *)state, init,
+                       total);
     return hipGetLastError();
 }
 

@@ -293,13 +293,12 @@ def test_outcoords_total_is_optional():
 
 @pytest.mark.parametrize("shape,p", [([40, 700, 20], 0.02), ([64, 1024, 70], 0.05), ([3, 21, 9], 0.5),
                                      ([500, 599, 8], 0.01), ([10, 30, 400], 0.05), ([12, 20, 250], 0.05),
-                                     ([6, 20, 1100], 0.02)])
+                                     ([6, 20, 1100], 0.02), ([900, 700, 4], 0.01)])
 def test_outcoords_scan_over_many_workgroups(shape, p):
-    """The scan of the per-column counts runs inside the count kernel, across its workgroups of 64 to 512
-    columns: grids of one workgroup, of hundreds (look-back over several windows of 64 predecessors), with
-    one, three and eight batches of 64 columns per workgroup (one grid ends inside a batch), and output
-    columns of 125, 200 and 550 bins (two and four masks per column kept; none beyond 512 bins), twice in a row on
-    the same scratch, against numpy's cumsum and the active set of a dense convolution."""
+    """Per-column counts and their one-pass scan (tiles of 2048 columns that look back over their
+    predecessors): grids of one tile, of tens and of more than 64 tiles (several look-back windows), ragged
+    ends, and output columns of 125, 200 and 550 bins (two and four masks per column kept; none beyond 512
+    bins), twice in a row on the same scratch, against numpy's cumsum and the active set of a dense convolution."""
     import ctypes as C
     from sphconv_amd import _lib as L
     rng = np.random.default_rng(shape[1])
