@@ -686,10 +686,14 @@ inline long scan_state_ints(long ncol) { return (long)(sph_scan::state_bytes(nco
 // 2048 workgroups of 64 columns, 31 us with 256 of 512 columns, against 19 us here + 6 us of scan).
 // `masks` (O2 <= 512 only, else null) keeps each column's bin masks for the fill kernel.
 __global__ __launch_bounds__(kCountThreads) void outcoords_count_kernel(OutArgs a, int32_t *counts,
-                                                                        unsigned long long *masks)
+                                                                        unsigned long long *masks, int *scan_state,
+                                                                        int scan_state_n)
 {
     const int ncol = a.B * a.O.n0 * a.O.n1;
     const int tid = threadIdx.x;
+    // the scan that follows on the stream finds its state cleared (saves the launch of a fill kernel)
+    if (blockIdx.x == 0)
+        for (int i = tid; i < scan_state_n; i += kCountThreads) scan_state[i] = 0;
     const int part = tid % kColLanes, cl = tid / kColLanes;
     const int oc = blockIdx.x * kCountCols + cl;
     if (oc >= ncol) return; // whole 16-lane groups leave together
@@ -994,11 +998,13 @@ static int outcoords_count(const char *who, const int32_t *z_idx, const int32_t 
     const long ncol = (long)g->B * g->O[0] * g->O[1];
     const unsigned nblocks = (unsigned)((ncol + kCountCols - 1) / kCountCols);
     hipLaunchKernelGGL(outcoords_count_kernel, dim3(nblocks), dim3(kCountThreads), 0, (hipStream_t)stream,
-                       out_args(z_idx, z_ptr, in_rows, g), oz_ptr, outcoords_masks(g, scratch));
+                       out_args(z_idx, z_ptr, in_rows, g), oz_ptr, outcoords_masks(g, scratch), (int *)scratch,
+                       sph_scan::state_ints(ncol));
     int rc = sph_check_launch(who);
     if (rc) return rc;
     // counts -> inclusive scan in place; the last tile also writes the row count
-    hipError_t e = sph_scan::launch<sph_scan::Plus, true>(oz_ptr, oz_ptr, ncol, scratch, 0, (hipStream_t)stream, total);
+    hipError_t e = sph_scan::launch<sph_scan::Plus, true>(oz_ptr, oz_ptr, ncol, scratch, 0, (hipStream_t)stream, total,
+                                                          /*clear_state=*/false);
     if (e != hipSuccess) {
         sph_set_error("%s: scan: %s", who, hipGetErrorString(e));
         return SPH_ERR_LAUNCH;

@@ -144,14 +144,19 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(const int32_t *in, int32
     }
 }
 
+// ints of the state that must be zero when the scan kernel starts
+inline int state_ints(long n) { return 2 + 2 * tiles(n > 0 ? n : 1); }
+
 // Enqueues the scan of n elements on st; state: state_bytes(n) bytes of device memory, 8-byte aligned.
+// clear_state = false: a kernel enqueued before on the same stream has already zeroed the first state_ints(n) ints.
 template <class OP, bool INCLUSIVE>
 inline hipError_t launch(const int32_t *in, int32_t *out, long n, void *state, int init, hipStream_t st,
-                         int32_t *total = nullptr)
+                         int32_t *total = nullptr, bool clear_state = true)
 {
     if (n <= 0) return hipSuccess;
-    const int nt = tiles(n), nints = 2 + 2 * nt;
-    hipLaunchKernelGGL(clear_state_kernel, dim3((nints + 255) / 256), dim3(256), 0, st, (int *)state, nints);
+    const int nt = tiles(n), nints = state_ints(n);
+    if (clear_state)
+        hipLaunchKernelGGL(clear_state_kernel, dim3((nints + 255) / 256), dim3(256), 0, st, (int *)state, nints);
     hipLaunchKernelGGL((scan_kernel<OP, INCLUSIVE>), dim3(nt), dim3(kThreads), 0, st, in, out, n, (int *)state, init,
                        total);
     return hipGetLastError();
