@@ -286,19 +286,36 @@ def test_wgrad_channel_blocks_and_chunks(dtype, ic, oc, subm):
     assert (np.abs(wide.double().cpu().numpy() - ref) <= 1e-5 * mag + 1e-6).all()
 
 
-def test_fused_epilogue_scale_shift_relu():
-    case = _random_case(41, True)
+@pytest.mark.parametrize("dtype,ic,oc,subm", [(torch.float32, 16, 32, True), (torch.float16, 32, 64, True),
+                                              (torch.bfloat16, 64, 64, False), (torch.float16, 20, 24, False),
+                                              (torch.float32, 5, 7, True)])
+def test_fused_epilogue_scale_shift_relu(dtype, ic, oc, subm):
+    """y = relu(acc * scale[c] + shift[c]) in the convolution's store, against the ORACLE's accumulator with the
+    affine and the ReLU applied in float64 (fast and general kernels, submanifold and strided books, with either
+    of scale / shift missing and without ReLU), and against the unfused device result."""
+    case = _random_case(41 + ic, subm)
     rng = np.random.default_rng(7)
-    n = case["sidx"].shape[0]
-    feat = rng.standard_normal((n, 16)).astype(np.float32)
-    w = _weights(rng, 27, 16, 32)
-    scale = (rng.random(32) + 0.5).astype(np.float32)
-    shift = rng.standard_normal(32).astype(np.float32)
+    n, m = case["sidx"].shape[0], case["book"].out_rows
+    feat = torch.tensor(rng.standard_normal((n, ic)).astype(np.float32)).to(dtype)
+    w = torch.tensor(_weights(rng, 27, ic, oc)).to(dtype)
+    scale = (rng.random(oc) + 0.5).astype(np.float32)
+    shift = rng.standard_normal(oc).astype(np.float32)
     book = case["book"]
-    plain = ext.rule_conv(G.t(feat), G.t(w), book, None, n)
-    fused = ext.rule_conv(G.t(feat), G.t(w), book, None, n, scale=G.t(scale), shift=G.t(shift), relu=True)
-    want = torch.relu(plain * G.t(scale) + G.t(shift))
-    torch.testing.assert_close(fused, want, rtol=1e-6, atol=1e-6)
+    acc = _oracle_fwd(case, feat.float().numpy(), w.float().numpy()).astype(np.float64)   # on the rounded inputs
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-3 * max(1.0, np.abs(acc).max()))
+    fd, wd = feat.to(G.DEV), w.to(G.DEV)
+    for use_scale, use_shift, relu in ((True, True, True), (True, False, False), (False, True, True), (True, True, False)):
+        want = acc * (scale if use_scale else 1.0) + (shift if use_shift else 0.0)
+        if relu:
+            want = np.maximum(want, 0.0)
+        got = ext.rule_conv(fd, wd, book, None, m, scale=G.t(scale) if use_scale else None,
+                            shift=G.t(shift) if use_shift else None, relu=relu)
+        assert got.dtype == dtype
+        np.testing.assert_allclose(got.double().cpu().numpy(), want, **tol)
+    if dtype == torch.float32:
+        plain = ext.rule_conv(fd, wd, book, None, m)
+        fused = ext.rule_conv(fd, wd, book, None, m, scale=G.t(scale), shift=G.t(shift), relu=True)
+        torch.testing.assert_close(fused, torch.relu(plain * G.t(scale) + G.t(shift)), rtol=1e-6, atol=1e-6)
 
 
 def test_stable_case_extreme_weights():
