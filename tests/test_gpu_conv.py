@@ -248,6 +248,7 @@ def test_half_backward(dtype):
     (torch.float16, 8, 24), (torch.float16, 40, 64), (torch.float16, 16, 32),
     (torch.bfloat16, 128, 64), (torch.bfloat16, 64, 128), (torch.bfloat16, 96, 48),
     (torch.float32, 72, 40), (torch.float32, 128, 128), (torch.float32, 4, 12),
+    (torch.float16, 6, 10), (torch.bfloat16, 3, 17),      # rows that are no whole 16-byte chunks: the general kernel
 ])
 @pytest.mark.parametrize("subm", [True, False])
 def test_wgrad_channel_blocks_and_chunks(dtype, ic, oc, subm):
