@@ -302,12 +302,24 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
 
     const int ngrp = a.book.tile_ngrp[tile];
     const long gb0 = (long)tile * a.cap;
-    const int32_t *gat = a.book.grp_gather + gb0 * SPH_GROUP;
-    const int32_t *own = a.book.grp_owner + gb0 * SPH_GROUP;
-    const int32_t *gk = a.book.grp_k + gb0;
+    // Every load of the loop goes through a buffer descriptor: the address is a scalar base plus a 32-bit lane
+    // offset (plus a scalar offset for the weight's kernel offset), so no load costs 64-bit vector arithmetic,
+    // and a read beyond the array returns zeros instead of faulting.  (The launcher sends arrays of 4 GiB or more
+    // to the general kernel.)
+    constexpr int kRsrcFlags = 0x00020000; // raw buffer, 32-bit data format
+    const __amdgpu_buffer_rsrc_t r_gat = __builtin_amdgcn_make_buffer_rsrc((void *)(a.book.grp_gather + gb0 * SPH_GROUP), 0,
+                                                                           a.cap * SPH_GROUP * 4, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t r_own = __builtin_amdgcn_make_buffer_rsrc((void *)(a.book.grp_owner + gb0 * SPH_GROUP), 0,
+                                                                           a.cap * SPH_GROUP * 4, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t r_gk = __builtin_amdgcn_make_buffer_rsrc((void *)(a.book.grp_k + gb0), 0, a.cap * 4, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t r_feat = __builtin_amdgcn_make_buffer_rsrc((void *)a.feat, 0, a.feat_rows * a.row_bytes, kRsrcFlags);
     // weight fragment of (offset k, step st, column tile c): k*NS*nwtot + st*nwtot + c  (1 KiB each)
-    const char *wlane = a.wp + ((long)(wave * CT)) * (kWave * 16) + lane * 16;
-    const long wstep = (long)nwtot * (kWave * 16);
+    const int wstep = nwtot * (kWave * 16);
+    const __amdgpu_buffer_rsrc_t r_w = __builtin_amdgcn_make_buffer_rsrc((void *)a.wp, 0, a.book.KV * NS * wstep, kRsrcFlags);
+    int woff[NS]; // lane offset of the wave's first column tile at step st
+#pragma unroll
+    for (int st = 0; st < NS; st++) woff[st] = st * wstep + (wave * CT) * (kWave * 16) + lane * 16;
+    const int lane_chunk = (lane >> 4) * 16;
 
     // Every load below is unconditional and straight-line (indices are clamped to
     // memory that is always allocated, results of invalid slots are discarded by
@@ -319,9 +331,9 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
     auto load_meta = [&](int g0, int &gi, int &ow, int &kk) {
         // one load each: lane l holds entry l%16 of group g0 + l/16; lanes 0..3 hold the offsets
         const int gs = min(g0, a.cap - kBlk); // stay inside this tile's capacity
-        gi = gat[(long)gs * SPH_GROUP + lane];
-        ow = own[(long)gs * SPH_GROUP + lane];
-        kk = gk[gs + (lane & (kBlk - 1))];
+        gi = __builtin_amdgcn_raw_buffer_load_b32(r_gat, lane * 4, gs * (SPH_GROUP * 4), 0);
+        ow = __builtin_amdgcn_raw_buffer_load_b32(r_own, lane * 4, gs * (SPH_GROUP * 4), 0);
+        kk = __builtin_amdgcn_raw_buffer_load_b32(r_gk, (lane & (kBlk - 1)) * 4, gs * 4, 0);
     };
     auto finish_meta = [&](int g0, int &gi, int &ow, int &kk) {
         const bool inside = g0 <= a.cap - kBlk;
@@ -337,19 +349,18 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
     // used, not here -- a select on the loaded value would stall the wave on the load.
     auto load_a = [&](int gi_blk, int u, int4v (&fa)[NS]) {
         const int in_row = __shfl(gi_blk, u * SPH_GROUP + (lane & 15), kWave);
-        const char *row = a.feat + (long)max(in_row, 0) * a.row_bytes;
+        const int row = max(in_row, 0) * a.row_bytes + lane_chunk;   // a row shorter than the step: the tail is the next row's, masked later
 #pragma unroll
-        for (int st = 0; st < NS; st++) {
-            const int off = st * 64 + (lane >> 4) * 16;
-            fa[st] = *(const int4v *)(row + (off < a.row_bytes ? off : 0));
-        }
+        for (int st = 0; st < NS; st++)
+            fa[st] = __builtin_bit_cast(int4v, __builtin_amdgcn_raw_buffer_load_b128(r_feat, row + st * 64, 0, 0));
     };
     auto load_w = [&](int k, int4v (&fw)[NS][CT]) {
-        const char *wk = wlane + (long)k * NS * wstep;
+        const int wk = k * (NS * wstep); // scalar
 #pragma unroll
         for (int st = 0; st < NS; st++)
 #pragma unroll
-            for (int c = 0; c < CT; c++) fw[st][c] = *(const int4v *)(wk + st * wstep + (long)c * (kWave * 16));
+            for (int c = 0; c < CT; c++)
+                fw[st][c] = __builtin_bit_cast(int4v, __builtin_amdgcn_raw_buffer_load_b128(r_w, woff[st] + c * (kWave * 16), wk, 0));
     };
     // Accumulator address of a pair: its owner's row, or the scratch row behind the tile for
     // a padding slot (which multiplies whatever row 0 holds): no branch, no select on data.
@@ -1587,7 +1598,9 @@ int launch_conv(const ConvArgs &a, int ntiles, hipStream_t st)
         if (a.nsteps == 1) return launch_conv_rows_ct<DT, 1>(a, NW, ntiles, st);
         return launch_conv_rows_ct<DT, 2>(a, NW, ntiles, st);
     }
-    if (a.aligned_in && a.feat_rows > 0) {
+    // the one-wave-per-tile kernel addresses the feature array through a buffer descriptor with 32-bit offsets
+    const bool small = (double)a.feat_rows * a.row_bytes < 2147483648.0;
+    if (a.aligned_in && a.feat_rows > 0 && small) {
         switch (a.nsteps) {
         case 1: return launch_conv_wave_ct<DT, 1>(a, NW, ntiles, st);
         case 2: return launch_conv_wave_ct<DT, 2>(a, NW, ntiles, st);
@@ -1595,7 +1608,7 @@ int launch_conv(const ConvArgs &a, int ntiles, hipStream_t st)
         default: break;
         }
     }
-    return launch_conv_ns<DT, NW, 0>(a, ntiles, st); // rows not a multiple of 16 bytes, or more than 256 bytes
+    return launch_conv_ns<DT, NW, 0>(a, ntiles, st); // rows not a multiple of 16 bytes, or more than 256 bytes, or 2 GiB of them
 }
 
 template <sph_dtype DT>
