@@ -690,3 +690,34 @@ def test_fp32_master_weight_gets_an_fp32_gradient():
     assert wide.abs().max() > 65504          # the case does leave fp16's range
     narrow = ext.rule_conv_d_weight(feat.detach(), up, case["book"], None)
     assert torch.isinf(narrow).any()
+
+
+def test_feature_array_of_two_gib_takes_the_general_kernel():
+    """The one-wave-per-tile kernel addresses the features with 32-bit offsets; an array of 2 GiB or more goes to
+    the general kernel, whose 64-bit addressing (and the by-row kernels') is checked here with a book that gathers
+    from the array's end."""
+    case = _random_case(91, True)
+    rng = np.random.default_rng(3)
+    n = case["sidx"].shape[0]
+    feat = rng.standard_normal((n, 64)).astype(np.float32)
+    w = _weights(rng, 27, 64, 64)
+    book = case["book"]
+    want = _oracle_fwd(case, torch.tensor(feat).half().float().numpy(), torch.tensor(w).half().float().numpy())
+    small = ext.rule_conv(G.t(feat).half(), G.t(w).half(), book, None, n)
+    np.testing.assert_allclose(small.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2)
+    rows = (1 << 24) + 4096                       # x 128 bytes = 2.0 GiB + 512 KiB
+    base = rows - n
+    big = torch.zeros((rows, 64), dtype=torch.float16, device=G.DEV)
+    big[base:] = G.t(feat).half()
+    tables = [book.fwd.grp_gather] + ([book.fwd.tile_nbr] if book.fwd.by_row else [])   # both forms name gathered rows
+    keep = [t.clone() for t in tables]
+    try:
+        for t, k in zip(tables, keep):
+            t.copy_(torch.where(k >= 0, k + base, k))
+        packed = ext._packed_weight(G.t(w).half(), False)
+        out = ext._apply(big, packed, 64, 64, book.fwd)
+    finally:
+        for t, k in zip(tables, keep):
+            t.copy_(k)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(out.float(), small.float(), rtol=1e-3, atol=1e-3)
