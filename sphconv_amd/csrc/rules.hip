@@ -151,14 +151,27 @@ __device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int t
     }
     if (!book.grp_gather) return; // the caller keeps the pairs by row only: no groups, and no group counts either
 
-    for (int k = wave; k < KV; k += kWaves) {
-        int r_lo = lane, r_hi = kWave + lane;
-        unsigned long long m0 = __ballot(r_lo < nrows && nbr[r_lo * KV + k] >= 0);
-        unsigned long long m1 = __ballot(r_hi < nrows && nbr[r_hi * KV + k] >= 0);
-        if (lane == 0) {
-            sc.mask[k][0] = m0;
-            sc.mask[k][1] = m1;
-            sc.cnt[k] = __popcll(m0) + __popcll(m1);
+    // a wave takes every kWaves-th offset, eight of them per round with all their table reads in flight together
+    // (one LDS round trip per round instead of one per offset)
+    constexpr int kEmitBatch = 8;
+    for (int kb = wave; kb < KV; kb += kWaves * kEmitBatch) {
+        int v_lo[kEmitBatch], v_hi[kEmitBatch];
+#pragma unroll
+        for (int q = 0; q < kEmitBatch; q++) {
+            const int k = min(kb + q * kWaves, KV - 1);
+            v_lo[q] = nbr[lane * KV + k];
+            v_hi[q] = nbr[(kWave + lane) * KV + k];
+        }
+#pragma unroll
+        for (int q = 0; q < kEmitBatch; q++) {
+            const int k = kb + q * kWaves;
+            const unsigned long long m0 = __ballot(lane < nrows && v_lo[q] >= 0);
+            const unsigned long long m1 = __ballot(kWave + lane < nrows && v_hi[q] >= 0);
+            if (lane == 0 && k < KV) {
+                sc.mask[k][0] = m0;
+                sc.mask[k][1] = m1;
+                sc.cnt[k] = __popcll(m0) + __popcll(m1);
+            }
         }
     }
     __syncthreads();
@@ -191,20 +204,42 @@ __device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int t
         book.tile_koff[(long)tile * (KV + 1) + k] = (uint16_t)sc.goff[k];
     const int ngrp = sc.goff[KV];
     const long gbase_tile = (long)tile * cap;
-    for (int slot = tid; slot < ngrp * SPH_GROUP; slot += kThreads) {
-        const int g = slot / SPH_GROUP;
-        const int k = sc.gk[g];
-        const int j = (g - sc.goff[k]) * SPH_GROUP + (slot & (SPH_GROUP - 1));
-        int gat = -1, own = -1;
-        if (j < sc.cnt[k]) {
-            const unsigned long long m0 = sc.mask[k][0];
-            const int c0 = __popcll(m0);
-            const int row = j < c0 ? select_bit(m0, j) : 64 + select_bit(sc.mask[k][1], j - c0);
-            gat = nbr[row * KV + k];
-            own = r0 + row;
+    // a thread's slots (slot, slot + kThreads, ...) three at a time: every step of the chain offset -> counts and
+    // masks -> row -> table entry is one LDS round trip for the three together
+    constexpr int kEmitSlots = 3;
+    const int nslots = ngrp * SPH_GROUP;
+    for (int s0 = tid; s0 < nslots; s0 += kThreads * kEmitSlots) {
+        int kq[kEmitSlots], jq[kEmitSlots], row[kEmitSlots], gat[kEmitSlots];
+        bool live[kEmitSlots];
+#pragma unroll
+        for (int q = 0; q < kEmitSlots; q++) {
+            const int slot = min(s0 + q * kThreads, nslots - 1);
+            kq[q] = sc.gk[slot / SPH_GROUP];
         }
-        book.grp_gather[gbase_tile * SPH_GROUP + slot] = gat;
-        book.grp_owner[gbase_tile * SPH_GROUP + slot] = own;
+#pragma unroll
+        for (int q = 0; q < kEmitSlots; q++) {
+            const int slot = min(s0 + q * kThreads, nslots - 1);
+            jq[q] = (slot / SPH_GROUP - sc.goff[kq[q]]) * SPH_GROUP + (slot & (SPH_GROUP - 1));
+            live[q] = jq[q] < sc.cnt[kq[q]];
+        }
+#pragma unroll
+        for (int q = 0; q < kEmitSlots; q++) {
+            const unsigned long long m0 = sc.mask[kq[q]][0], m1 = sc.mask[kq[q]][1];
+            const int c0 = __popcll(m0);
+            const int j = live[q] ? jq[q] : 0;
+            row[q] = j < c0 ? select_bit(m0, j) : 64 + select_bit(m1, min(j - c0, 63));
+            row[q] = min(row[q], R - 1);
+        }
+#pragma unroll
+        for (int q = 0; q < kEmitSlots; q++) gat[q] = nbr[row[q] * KV + kq[q]];
+#pragma unroll
+        for (int q = 0; q < kEmitSlots; q++) {
+            const int slot = s0 + q * kThreads;
+            if (slot < nslots) {
+                book.grp_gather[gbase_tile * SPH_GROUP + slot] = live[q] ? gat[q] : -1;
+                book.grp_owner[gbase_tile * SPH_GROUP + slot] = live[q] ? r0 + row[q] : -1;
+            }
+        }
     }
     for (int g = tid; g < ngrp; g += kThreads) book.grp_k[gbase_tile + g] = sc.gk[g];
 }
