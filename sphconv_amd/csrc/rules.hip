@@ -29,6 +29,16 @@ struct ConvParams {
     int p0, p1, p2;
 };
 
+// Barrier for data exchanged through LDS only.  __syncthreads() also waits for every global load and store of
+// the thread that is still in flight (a full memory round trip each time one is pending); the rule kernels
+// share nothing through global memory inside a workgroup, so their barriers order LDS accesses alone.
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 __device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
 // Row range [start, end) of column c, clamped to [0, rows] so that inconsistent
@@ -58,14 +68,14 @@ __device__ int block_upper_bound(const int32_t *a, int n, int target, int max_sp
         int val = (pos < hi) ? a[pos] : 0x7fffffff; // positions >= hi are known to exceed
         int first = (val > target) ? tid : kThreads;
         if (tid == 0) *s_tmp = kThreads;
-        __syncthreads();
+        lds_barrier();
         // one LDS atomic per wave: reduce to the wave's smallest index first
 #pragma unroll
         for (int off = kWave / 2; off > 0; off >>= 1) first = min(first, __shfl_xor(first, off, kWave));
         if ((tid & (kWave - 1)) == 0 && first < kThreads) atomicMin(s_tmp, first);
-        __syncthreads();
+        lds_barrier();
         int f = *s_tmp;
-        __syncthreads();
+        lds_barrier();
         if (f == kThreads) {
             lo = lo + (kThreads - 1) * step + 1;
         } else {
@@ -81,63 +91,64 @@ __device__ int block_upper_bound(const int32_t *a, int n, int target, int max_sp
 
 // ---------------------------------------------------------------------------
 // Shared tail of the book builders: the block holds, in LDS, a table
-// nbr[row_local * KV + k] = gathered row or -1 for the `nrows` rows of tile
-// `tile` (first row r0).  Emits the tile's groups: per k, rows in ascending
-// order, 16 per group, last group padded with -1.
-//   pass 1: per k a 128-bit occupancy mask of the rows (wave ballots) and its count;
-//   scan  : first group of every k;
-//   pass 2: one thread per output SLOT finds its k and its rank in the k-list,
-//           selects the rank-th set bit of the mask and stores -- consecutive
-//           threads store consecutive slots, so the book is written coalesced.
+// nbr[row_local * KV + k] = gathered row or -1 for the R rows of tile `tile`
+// (first row r0; rows behind the tile's last one hold -1).  Emits the tile's
+// groups: per k, rows in ascending order, 16 per group, last group padded with -1.
+//   pass 1: a wave takes an offset k: two ballots over the column k of the table
+//           give every row with a pair its rank in the k-list, and the row writes
+//           its number into the list's place in LDS (sel[k][rank]);
+//   scan  : first group of every k, and one descriptor word per group;
+//   pass 2: one thread per output SLOT reads its group's descriptor, the row at its
+//           rank and the row's table entry, and stores -- consecutive threads store
+//           consecutive slots, so the book is written coalesced.
+// The rule kernels are bound by the number of vector instructions they issue (three
+// waves per SIMD, each instruction four cycles), not by latency: every step above is
+// a handful of instructions per item.
 // ---------------------------------------------------------------------------
-// Lives in dynamic LDS behind the neighbour table, sized by the kernel volume (a 3x3x3 kernel needs 0.9 KB
-// where the largest volume would need 4 KB: one more workgroup per CU).
+// Lives in dynamic LDS behind the neighbour table, sized by the kernel volume (a 3x3x3 kernel needs 4.5 KB
+// where the largest volume needs 21 KB).
 struct EmitScratch {
-    unsigned long long (*mask)[R / 64]; // [KV]
-    int *cnt;                           // [KV]
-    int *goff;                          // [KV + 1]
-    unsigned char *gk;                  // [KV * (R / SPH_GROUP)]
+    int *cnt;           // [KV] pairs of offset k
+    int *goff;          // [KV + 1] first group of offset k
+    int *ginfo;         // [KV * (R / SPH_GROUP)] per group: k | rank of its first slot << 8 | cnt[k] << 16
+    unsigned char *sel; // [KV][R] rows of offset k's list
 };
 __host__ __device__ inline size_t emit_scratch_bytes(int KV)
 {
-    const size_t b = (size_t)KV * (R / 64) * sizeof(unsigned long long) + (size_t)KV * sizeof(int) +
-                     (size_t)(KV + 1) * sizeof(int) + (size_t)KV * (R / SPH_GROUP);
+    const size_t b = (size_t)KV * sizeof(int) + (size_t)(KV + 1) * sizeof(int) +
+                     (size_t)KV * (R / SPH_GROUP) * sizeof(int) + (size_t)KV * R;
     return (b + 7) & ~(size_t)7;
 }
-// `base` must be 8-byte aligned.
+// `base` must be 4-byte aligned.
 __device__ __forceinline__ EmitScratch emit_scratch_at(void *base, int KV)
 {
     EmitScratch sc;
-    sc.mask = (unsigned long long (*)[R / 64])base;
-    sc.cnt = (int *)(sc.mask + KV);
+    sc.cnt = (int *)base;
     sc.goff = sc.cnt + KV;
-    sc.gk = (unsigned char *)(sc.goff + KV + 1);
+    sc.ginfo = sc.goff + KV + 1;
+    sc.sel = (unsigned char *)(sc.ginfo + KV * (R / SPH_GROUP));
     return sc;
 }
 
-// Position of the j-th (0-based) set bit of m; m must have more than j bits set.
-__device__ __forceinline__ int select_bit(unsigned long long m, int j)
+// Inclusive sum over the wave's 64 lanes through the data-parallel-primitive lane shifts of the vector ALU
+// (four shifts inside a row of 16 lanes, then lane 15 and lane 31 broadcast into the rows behind them):
+// no LDS round trip per step as a shuffle has.
+__device__ __forceinline__ int wave_inclusive_sum(int x)
 {
-    int base = 0;
-#pragma unroll
-    for (int w = 32; w >= 1; w >>= 1) {
-        unsigned long long low = m & ((1ull << w) - 1ull);
-        int c = __popcll(low);
-        if (j >= c) {
-            j -= c;
-            m >>= w;
-            base += w;
-        } else {
-            m = low;
-        }
-    }
-    return base;
+    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, false); // row_shr:1
+    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, false); // row_shr:2
+    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, false); // row_shr:4
+    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, false); // row_shr:8
+    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, false); // row_bcast:15 into rows 1 and 3
+    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, false); // row_bcast:31 into rows 2 and 3
+    return x;
 }
 
 __device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int tile, int cap,
                             const EmitScratch &sc, const sph_book &book)
 {
-    static_assert(R == 128, "the occupancy masks assume 128 rows per tile");
+    static_assert(R == 128 && kWave == 64, "two ballots cover a tile's rows");
+    static_assert(R / SPH_GROUP <= 8 && R <= 128, "a group descriptor packs k, a rank and a count into 8 bits each");
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
@@ -146,7 +157,7 @@ __device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int t
         int32_t *dst = book.tile_nbr + (long)tile * KV * R;
         for (int i = tid; i < KV * R; i += kThreads) {
             const int k = i / R, r = i - k * R;
-            dst[i] = r < nrows ? nbr[r * KV + k] : -1;
+            dst[i] = nbr[r * KV + k];
         }
     }
     if (!book.grp_gather) return; // the caller keeps the pairs by row only: no groups, and no group counts either
@@ -165,83 +176,73 @@ __device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int t
 #pragma unroll
         for (int q = 0; q < kEmitBatch; q++) {
             const int k = kb + q * kWaves;
-            const unsigned long long m0 = __ballot(lane < nrows && v_lo[q] >= 0);
-            const unsigned long long m1 = __ballot(kWave + lane < nrows && v_hi[q] >= 0);
-            if (lane == 0 && k < KV) {
-                sc.mask[k][0] = m0;
-                sc.mask[k][1] = m1;
-                sc.cnt[k] = __popcll(m0) + __popcll(m1);
+            if (k < KV) { // the same for the whole wave
+                const unsigned long long m0 = __ballot(v_lo[q] >= 0), m1 = __ballot(v_hi[q] >= 0);
+                const int c0 = __popcll(m0);
+                // set bits below this lane = the row's rank among the rows of its half
+                const int b0 = __builtin_amdgcn_mbcnt_hi((unsigned)(m0 >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m0, 0));
+                const int b1 = __builtin_amdgcn_mbcnt_hi((unsigned)(m1 >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m1, 0));
+                unsigned char *list = sc.sel + k * R;
+                if (v_lo[q] >= 0) list[b0] = (unsigned char)lane;
+                if (v_hi[q] >= 0) list[c0 + b1] = (unsigned char)(kWave + lane);
+                if (lane == 0) sc.cnt[k] = c0 + __popcll(m1);
             }
         }
     }
-    __syncthreads();
+    lds_barrier();
     if (wave == 0) {
         // exclusive scan of the per-offset group counts by one wave (KV <= 128: two passes)
         int carry = 0;
         for (int k0 = 0; k0 < KV; k0 += kWave) {
-            int k = k0 + lane;
-            int v = (k < KV) ? (sc.cnt[k] + SPH_GROUP - 1) / SPH_GROUP : 0;
-            int incl = v;
-#pragma unroll
-            for (int off = 1; off < kWave; off <<= 1) {
-                int t = __shfl_up(incl, off, kWave);
-                if (lane >= off) incl += t;
-            }
+            const int k = k0 + lane;
+            const int c = (k < KV) ? sc.cnt[k] : 0;
+            const int v = (c + SPH_GROUP - 1) / SPH_GROUP;
+            const int incl = wave_inclusive_sum(v);
             if (k < KV) {
-                sc.goff[k] = carry + incl - v;
-                for (int g = 0; g < v; g++) sc.gk[carry + incl - v + g] = (unsigned char)k;
+                const int first = carry + incl - v;
+                sc.goff[k] = first;
+                for (int g = 0; g < v; g++) sc.ginfo[first + g] = k | (g * SPH_GROUP) << 8 | c << 16;
             }
-            carry += __shfl(incl, kWave - 1, kWave);
+            carry += __builtin_amdgcn_readlane(incl, kWave - 1);
         }
         if (lane == 0) {
             sc.goff[KV] = carry;
             book.tile_ngrp[tile] = carry;
         }
     }
-    __syncthreads();
+    lds_barrier();
 
     for (int k = tid; k <= KV; k += kThreads)
         book.tile_koff[(long)tile * (KV + 1) + k] = (uint16_t)sc.goff[k];
     const int ngrp = sc.goff[KV];
     const long gbase_tile = (long)tile * cap;
-    // a thread's slots (slot, slot + kThreads, ...) three at a time: every step of the chain offset -> counts and
-    // masks -> row -> table entry is one LDS round trip for the three together
-    constexpr int kEmitSlots = 3;
+    int32_t *out_gather = book.grp_gather + gbase_tile * SPH_GROUP, *out_owner = book.grp_owner + gbase_tile * SPH_GROUP;
+    // a thread's slots (slot, slot + kThreads, ...) four at a time: every step of the chain descriptor -> row ->
+    // table entry is one LDS round trip for the four together
+    constexpr int kEmitSlots = 4;
     const int nslots = ngrp * SPH_GROUP;
     for (int s0 = tid; s0 < nslots; s0 += kThreads * kEmitSlots) {
-        int kq[kEmitSlots], jq[kEmitSlots], row[kEmitSlots], gat[kEmitSlots];
-        bool live[kEmitSlots];
+        int info[kEmitSlots], row[kEmitSlots], gat[kEmitSlots];
+#pragma unroll
+        for (int q = 0; q < kEmitSlots; q++) info[q] = sc.ginfo[min(s0 + q * kThreads, nslots - 1) / SPH_GROUP];
 #pragma unroll
         for (int q = 0; q < kEmitSlots; q++) {
-            const int slot = min(s0 + q * kThreads, nslots - 1);
-            kq[q] = sc.gk[slot / SPH_GROUP];
+            // s0 and s0 + q * kThreads share their place in the group (kThreads is a multiple of the group size)
+            const int k = info[q] & 0xff, j = ((info[q] >> 8) & 0xff) + (tid & (SPH_GROUP - 1));
+            row[q] = j < (info[q] >> 16) ? sc.sel[k * R + j] : -1;
         }
 #pragma unroll
-        for (int q = 0; q < kEmitSlots; q++) {
-            const int slot = min(s0 + q * kThreads, nslots - 1);
-            jq[q] = (slot / SPH_GROUP - sc.goff[kq[q]]) * SPH_GROUP + (slot & (SPH_GROUP - 1));
-            live[q] = jq[q] < sc.cnt[kq[q]];
-        }
-#pragma unroll
-        for (int q = 0; q < kEmitSlots; q++) {
-            const unsigned long long m0 = sc.mask[kq[q]][0], m1 = sc.mask[kq[q]][1];
-            const int c0 = __popcll(m0);
-            const int j = live[q] ? jq[q] : 0;
-            row[q] = j < c0 ? select_bit(m0, j) : 64 + select_bit(m1, min(j - c0, 63));
-            row[q] = min(row[q], R - 1);
-        }
-#pragma unroll
-        for (int q = 0; q < kEmitSlots; q++) gat[q] = nbr[row[q] * KV + kq[q]];
+        for (int q = 0; q < kEmitSlots; q++) gat[q] = nbr[max(row[q], 0) * KV + (info[q] & 0xff)];
 #pragma unroll
         for (int q = 0; q < kEmitSlots; q++) {
             const int slot = s0 + q * kThreads;
             if (slot < nslots) {
-                book.grp_gather[gbase_tile * SPH_GROUP + slot] = live[q] ? gat[q] : -1;
-                book.grp_owner[gbase_tile * SPH_GROUP + slot] = live[q] ? r0 + row[q] : -1;
+                out_gather[slot] = row[q] >= 0 ? gat[q] : -1;
+                out_owner[slot] = row[q] >= 0 ? r0 + row[q] : -1;
             }
         }
     }
-    for (int g = tid; g < ngrp; g += kThreads) book.grp_k[gbase_tile + g] = sc.gk[g];
+    for (int g = tid; g < ngrp; g += kThreads) book.grp_k[gbase_tile + g] = sc.ginfo[g] & 0xff;
 }
 
 // ---------------------------------------------------------------------------
@@ -304,7 +305,7 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
 
     for (int i = tid; i < R * KV / 4; i += kThreads) ((int4 *)s_nbr)[i] = make_int4(-1, -1, -1, -1); // R * KV is a multiple of 4
     for (int i = tid; i < R; i += kThreads) s_col[i] = -1;
-    __syncthreads();
+    lds_barrier();
 
     // 1. rows -> columns.  The walk below tolerates starting early (columns before the
     // tile hold none of its rows), so the search stops once the window is below one
@@ -326,9 +327,9 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
             for (int r = max(p1, r0); r < min(p2, r1); r++) s_col[r - r0] = c + 1;
             if (c == last || c + 1 == last) s_flag = (p2 >= r1) || (last == q_ncol - 1);
         }
-        __syncthreads();
+        lds_barrier();
         done = s_flag != 0;
-        __syncthreads();
+        lds_barrier();
     }
     if (tid < nrows) {
         int c = s_col[tid];
@@ -341,7 +342,7 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
             s_z[tid] = my_z;
         }
     }
-    __syncthreads();
+    lds_barrier();
 
     // 2a. join through masks (long fibers).  The tile's rows share few columns, and every row of
     // a column would walk the same K0*K1 fibers of the other grid: walk each (column, k0, k1)
@@ -362,7 +363,7 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
             const unsigned long long bal = __ballot(head);
             if (lane == 0) s_bal[wave] = bal;
         }
-        __syncthreads();
+        lds_barrier();
         int ncols = 0;
         for (int w = 0; w < R / kWave; w++) ncols += __popcll(s_bal[w]);
         if (tid < R) {
@@ -372,7 +373,7 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
             s_cj[tid] = cj;
             if (head) s_rep[cj] = tid;
         }
-        __syncthreads();
+        lds_barrier();
         if (ncols > kMaskCols) ncols = 0; // short fibers after all: general join
         for (int it = tid; it < ncols * K01; it += kThreads) {
             const int k01 = it / ncols, cj = it - k01 * ncols;
@@ -414,7 +415,7 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
             s_cmask[it] = m;
             s_cstart[it] = st;
         }
-        __syncthreads();
+        lds_barrier();
         by_masks = s_bad == 0 && ncols > 0;
         const bool pow2_s2 = (a.cv.s2 & (a.cv.s2 - 1)) == 0;
         const int sh_s2 = __ffs(a.cv.s2) - 1;
@@ -535,7 +536,7 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
             }
         }
     }
-    __syncthreads();
+    lds_barrier();
 
     // 3. compaction
     emit_groups(s_nbr, nrows, r0, KV, tile, a.cap, emit_scratch_at(s_nbr + R * KV, KV), a.book);
@@ -550,8 +551,8 @@ __global__ __launch_bounds__(kThreads) void book_from_nbr_kernel(const int32_t *
     const int tile = blockIdx.x;
     const int r0 = tile * R;
     const int nrows = min(R, rows - r0);
-    for (int i = threadIdx.x; i < nrows * KV; i += kThreads) s_nbr[i] = nbr[(long)r0 * KV + i];
-    __syncthreads();
+    for (int i = threadIdx.x; i < R * KV; i += kThreads) s_nbr[i] = i < nrows * KV ? nbr[(long)r0 * KV + i] : -1;
+    lds_barrier();
     emit_groups(s_nbr, nrows, r0, KV, tile, cap, emit_scratch_at(s_nbr + R * KV, KV), book);
 }
 
