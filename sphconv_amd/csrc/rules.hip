@@ -56,26 +56,25 @@ __device__ __forceinline__ void fiber_range(const int32_t *ptr, int c, int rows,
 // round cuts the window by a factor of kThreads.  (Probes are scattered, one cache
 // line each, and cost far more in the vector memory path than the coalesced column
 // walk that follows; hence few probes and an early stop.)  max_span = 1 gives the
-// exact column.  s_tmp: one LDS int.  Must be called by the whole block.
-__device__ int block_upper_bound(const int32_t *a, int n, int target, int max_span, int *s_tmp)
+// exact column.  s_first: 2 * kWaves LDS ints (the rounds alternate between the halves,
+// so a round needs one barrier).  Must be called by the whole block.
+__device__ int block_upper_bound(const int32_t *a, int n, int target, int max_span, int *s_first)
 {
     int lo = 0, hi = n;
     const int tid = threadIdx.x;
-    while (hi - lo >= max_span) {
+    for (int round = 0; hi - lo >= max_span; round ^= 1) {
         int span = hi - lo;
         int step = (span + kThreads - 1) / kThreads;
         long pos = (long)lo + (long)tid * step;
         int val = (pos < hi) ? a[pos] : 0x7fffffff; // positions >= hi are known to exceed
-        int first = (val > target) ? tid : kThreads;
-        if (tid == 0) *s_tmp = kThreads;
+        // first probe above the target: per wave by a ballot, over the waves through LDS
+        const unsigned long long above = __ballot(val > target);
+        int *mine = s_first + round * kWaves;
+        if ((tid & (kWave - 1)) == 0) mine[tid / kWave] = above ? (tid & ~(kWave - 1)) + __ffsll((long long)above) - 1 : kThreads;
         lds_barrier();
-        // one LDS atomic per wave: reduce to the wave's smallest index first
+        int f = kThreads;
 #pragma unroll
-        for (int off = kWave / 2; off > 0; off >>= 1) first = min(first, __shfl_xor(first, off, kWave));
-        if ((tid & (kWave - 1)) == 0 && first < kThreads) atomicMin(s_tmp, first);
-        lds_barrier();
-        int f = *s_tmp;
-        lds_barrier();
+        for (int w = 0; w < kWaves; w++) f = min(f, mine[w]);
         if (f == kThreads) {
             lo = lo + (kThreads - 1) * step + 1;
         } else {
@@ -175,8 +174,8 @@ __device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int t
         }
 #pragma unroll
         for (int q = 0; q < kEmitBatch; q++) {
-            const int k = kb + q * kWaves;
-            if (k < KV) { // the same for the whole wave
+            const int k = min(kb + q * kWaves, KV - 1); // behind the last offset: the last one again, same values
+            {
                 const unsigned long long m0 = __ballot(v_lo[q] >= 0), m1 = __ballot(v_hi[q] >= 0);
                 const int c0 = __popcll(m0);
                 // set bits below this lane = the row's rank among the rows of its half
@@ -185,7 +184,7 @@ __device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int t
                 unsigned char *list = sc.sel + k * R;
                 if (v_lo[q] >= 0) list[b0] = (unsigned char)lane;
                 if (v_hi[q] >= 0) list[c0 + b1] = (unsigned char)(kWave + lane);
-                if (lane == 0) sc.cnt[k] = c0 + __popcll(m1);
+                sc.cnt[k] = c0 + __popcll(m1); // every lane the same value
             }
         }
     }
@@ -282,7 +281,7 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     extern __shared__ __attribute__((aligned(16))) int32_t s_nbr[]; // [R * KV]
     __shared__ int s_col[R];
     __shared__ int s_b[R], s_c0[R], s_c1[R], s_z[R];
-    __shared__ int s_tmp, s_flag;
+    __shared__ int s_first[2 * kWaves], s_flag[2];
 
     const int tid = threadIdx.x;
     if ((int)blockIdx.x >= a.tile_blocks) {
@@ -311,9 +310,9 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     // tile hold none of its rows), so the search stops once the window is below one
     // walk step: a single round of probes for grids of up to 131072 columns.
     constexpr int kWalk = 2 * kThreads; // columns per walk step, two consecutive ones per thread
-    int c_first = block_upper_bound(a.q_ptr, q_ncol, r0, kWalk, &s_tmp);
+    int c_first = block_upper_bound(a.q_ptr, q_ncol, r0, kWalk, s_first);
     bool done = (c_first >= q_ncol);
-    for (int cb = c_first; !done; cb += kWalk) {
+    for (int cb = c_first, step = 0; !done; cb += kWalk, step ^= 1) { // the steps alternate between two flags: one barrier each
         const int last = min(cb + kWalk - 1, q_ncol - 1);
         const int c = cb + 2 * tid;
         if (c <= last) {
@@ -325,11 +324,10 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
             if (p2 < p1) p2 = p1;
             for (int r = max(p0, r0); r < min(p1, r1); r++) s_col[r - r0] = c;
             for (int r = max(p1, r0); r < min(p2, r1); r++) s_col[r - r0] = c + 1;
-            if (c == last || c + 1 == last) s_flag = (p2 >= r1) || (last == q_ncol - 1);
+            if (c == last || c + 1 == last) s_flag[step] = (p2 >= r1) || (last == q_ncol - 1);
         }
         lds_barrier();
-        done = s_flag != 0;
-        lds_barrier();
+        done = s_flag[step] != 0;
     }
     if (tid < nrows) {
         int c = s_col[tid];
