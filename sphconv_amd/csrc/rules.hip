@@ -23,6 +23,25 @@ struct Grid3 {
     int n0, n1, n2;
 };
 
+// Division of a 32-bit unsigned number by a divisor fixed per launch: a multiplication and two shifts with
+// constants made on the host (Granlund and Montgomery's round-up method, exact for every 32-bit numerator),
+// where the compiler's division by a run-time value is some thirty instructions in a row.
+struct FastDiv {
+    uint32_t mul, sh1, sh2;
+};
+inline FastDiv fast_div(uint32_t d)
+{
+    uint32_t l = 0;
+    while ((1ull << l) < d) l++;
+    const uint32_t m = (uint32_t)((((1ull << l) - d) << 32) / d + 1);
+    return FastDiv{m, l < 1 ? l : 1, l < 1 ? 0 : l - 1};
+}
+__device__ __forceinline__ uint32_t div_by(uint32_t n, const FastDiv &f)
+{
+    const uint32_t t = __umulhi(f.mul, n);
+    return (t + ((n - t) >> f.sh1)) >> f.sh2;
+}
+
 struct ConvParams {
     int K0, K1, K2;
     int s0, s1, s2;
@@ -57,16 +76,21 @@ __device__ __forceinline__ void fiber_range(const int32_t *ptr, int c, int rows,
 // line each, and cost far more in the vector memory path than the coalesced column
 // walk that follows; hence few probes and an early stop.)  max_span = 1 gives the
 // exact column.  s_first: 2 * kWaves LDS ints (the rounds alternate between the halves,
-// so a round needs one barrier).  Must be called by the whole block.
-__device__ int block_upper_bound(const int32_t *a, int n, int target, int max_span, int *s_first)
+// so a round needs one barrier).  meanwhile() runs once, while the first round's probes are in flight,
+// and in front of a barrier: the place for LDS initialisation.  Must be called by the whole block.
+template <class F>
+__device__ int block_upper_bound(const int32_t *a, int n, int target, int max_span, int *s_first, F &&meanwhile)
 {
     int lo = 0, hi = n;
     const int tid = threadIdx.x;
+    bool first = true;
     for (int round = 0; hi - lo >= max_span; round ^= 1) {
         int span = hi - lo;
         int step = (span + kThreads - 1) / kThreads;
         long pos = (long)lo + (long)tid * step;
         int val = (pos < hi) ? a[pos] : 0x7fffffff; // positions >= hi are known to exceed
+        if (first) meanwhile();
+        first = false;
         // first probe above the target: per wave by a ballot, over the waves through LDS
         const unsigned long long above = __ballot(val > target);
         int *mine = s_first + round * kWaves;
@@ -84,6 +108,10 @@ __device__ int block_upper_bound(const int32_t *a, int n, int target, int max_sp
             hi = new_hi;
             lo = new_lo;
         }
+    }
+    if (first) { // no round at all
+        meanwhile();
+        lds_barrier();
     }
     return lo;
 }
@@ -269,6 +297,7 @@ struct BuildArgs {
     // gathered-side fibers are long (several entries on average) and their bins fit a 64-bit mask:
     // join through per-column occupancy masks instead of walking a fiber once per row
     int long_fibers;
+    FastDiv by_q1, by_q01; // division by Q.n1 and by Q.n0 * Q.n1
 };
 
 constexpr int kMaskCols = 32;  // distinct columns of a tile the mask join provides for
@@ -280,7 +309,6 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
 {
     extern __shared__ __attribute__((aligned(16))) int32_t s_nbr[]; // [R * KV]
     __shared__ int s_col[R];
-    __shared__ int s_b[R], s_c0[R], s_c1[R], s_z[R];
     __shared__ int s_first[2 * kWaves], s_flag[2];
 
     const int tid = threadIdx.x;
@@ -299,18 +327,20 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     const int nrows = r1 - r0;
     const int q_ncol = a.B * a.Q.n0 * a.Q.n1;
 
-    // the tile's own S2 coordinates do not depend on the column search: fetch them first
-    const int my_z = (tid < nrows) ? a.q_idx[r0 + tid] : 0;
-
-    for (int i = tid; i < R * KV / 4; i += kThreads) ((int4 *)s_nbr)[i] = make_int4(-1, -1, -1, -1); // R * KV is a multiple of 4
-    for (int i = tid; i < R; i += kThreads) s_col[i] = -1;
-    lds_barrier();
+    // the tile's own S2 coordinates do not depend on the column search: fetch them first.  A row belongs to
+    // the kThreads / R threads that share its number: each keeps the row's coordinates in registers.
+    static_assert(kThreads % R == 0, "a thread's items must share a row");
+    const int my_rl = tid & (R - 1);
+    const int my_zz = (my_rl < nrows) ? a.q_idx[r0 + my_rl] : 0;
 
     // 1. rows -> columns.  The walk below tolerates starting early (columns before the
     // tile hold none of its rows), so the search stops once the window is below one
     // walk step: a single round of probes for grids of up to 131072 columns.
     constexpr int kWalk = 2 * kThreads; // columns per walk step, two consecutive ones per thread
-    int c_first = block_upper_bound(a.q_ptr, q_ncol, r0, kWalk, s_first);
+    int c_first = block_upper_bound(a.q_ptr, q_ncol, r0, kWalk, s_first, [&]() {
+        for (int i = tid; i < R * KV / 4; i += kThreads) ((int4 *)s_nbr)[i] = make_int4(-1, -1, -1, -1); // R * KV is a multiple of 4
+        for (int i = tid; i < R; i += kThreads) s_col[i] = -1;
+    });
     bool done = (c_first >= q_ncol);
     for (int cb = c_first, step = 0; !done; cb += kWalk, step ^= 1) { // the steps alternate between two flags: one barrier each
         const int last = min(cb + kWalk - 1, q_ncol - 1);
@@ -329,18 +359,12 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
         lds_barrier();
         done = s_flag[step] != 0;
     }
-    if (tid < nrows) {
-        int c = s_col[tid];
-        if (c >= 0) {
-            int b = c / (a.Q.n0 * a.Q.n1);
-            int rem = c - b * (a.Q.n0 * a.Q.n1);
-            s_b[tid] = b;
-            s_c0[tid] = rem / a.Q.n1;
-            s_c1[tid] = rem % a.Q.n1;
-            s_z[tid] = my_z;
-        }
-    }
-    lds_barrier();
+    // the row's column -> (batch, S0, S1), by every thread for its own row
+    const int my_c = my_rl < nrows ? s_col[my_rl] : -1;
+    const bool my_ok = my_c >= 0;
+    const int my_b = (int)div_by((uint32_t)max(my_c, 0), a.by_q01);
+    const int my_rem = max(my_c, 0) - my_b * (a.Q.n0 * a.Q.n1);
+    const int my_c0 = (int)div_by((uint32_t)my_rem, a.by_q1), my_c1 = my_rem - my_c0 * a.Q.n1;
 
     // 2a. join through masks (long fibers).  The tile's rows share few columns, and every row of
     // a column would walk the same K0*K1 fibers of the other grid: walk each (column, k0, k1)
@@ -351,7 +375,14 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     if (a.long_fibers) {
         unsigned long long *s_cmask = (unsigned long long *)((char *)(s_nbr + R * KV) + emit_scratch_bytes(KV)); // [K01][ncols], ncols <= kMaskCols
         int *s_cstart = (int *)(s_cmask + kMaskCols * K01);
+        __shared__ int s_b[R], s_c0[R], s_c1[R], s_z[R];
         __shared__ int s_cj[R], s_rep[R], s_bad;
+        if (tid < R && my_ok) {
+            s_b[tid] = my_b;
+            s_c0[tid] = my_c0;
+            s_c1[tid] = my_c1;
+            s_z[tid] = my_zz;
+        }
         __shared__ unsigned long long s_bal[R / kWave];
         const int lane = tid & (kWave - 1), wave = tid / kWave;
         if (tid == 0) s_bad = 0;
@@ -453,15 +484,10 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     // kThreads is a multiple of R, so a thread meets the same row in every item: what depends on the row
     // only is fetched from LDS and multiplied once, and an item costs a handful of integer operations
     // (k0 = k01 / K1 by a 16-bit reciprocal, exact for the k01 < 256 that a kernel volume <= 128 allows)
-    static_assert(kThreads % R == 0, "a thread's items must share a row");
-    const int my_rl = tid & (R - 1);
-    const bool my_ok = my_rl < nrows && s_col[my_rl] >= 0;
-    const int my_rr = my_ok ? my_rl : 0;
-    const int my_zz = s_z[my_rr];
-    const int my_a0 = TRANSPOSED ? s_c0[my_rr] + a.cv.p0 : s_c0[my_rr] * a.cv.s0 - a.cv.p0;
-    const int my_a1 = TRANSPOSED ? s_c1[my_rr] + a.cv.p1 : s_c1[my_rr] * a.cv.s1 - a.cv.p1;
-    const int my_col0 = s_b[my_rr] * a.P.n0;
-    const int my_slot = my_rr * KV;
+    const int my_a0 = TRANSPOSED ? my_c0 + a.cv.p0 : my_c0 * a.cv.s0 - a.cv.p0;
+    const int my_a1 = TRANSPOSED ? my_c1 + a.cv.p1 : my_c1 * a.cv.s1 - a.cv.p1;
+    const int my_col0 = my_b * a.P.n0;
+    const int my_slot = my_rl * KV;
     const unsigned inv_k1 = (65536u + a.cv.K1 - 1) / a.cv.K1;
     const bool unit_stride = a.cv.s0 == 1 && a.cv.s1 == 1;
     const bool pow2_stride = (a.cv.s0 & (a.cv.s0 - 1)) == 0 && (a.cv.s1 & (a.cv.s1 - 1)) == 0;
@@ -933,6 +959,8 @@ static int rules_build(const char *who, const int32_t *z_idx, const int32_t *z_p
     }
     a.B = g->B;
     a.cv = conv_params(g);
+    a.by_q1 = fast_div((uint32_t)a.Q.n1);
+    a.by_q01 = fast_div((uint32_t)a.Q.n0 * (uint32_t)a.Q.n1);
     a.cap = sph_book_cap(KV);
     a.book = *book;
     const int nt = sph_book_tiles(book->rows);
