@@ -419,13 +419,24 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
     for (int i = lane; i < (R + 1) * CT * 4; i += kWave)
         *(int4v *)&s_acc[(i / (CT * 4)) * LDW + col0 + (i % (CT * 4)) * 4] = int4v{0, 0, 0, 0};
     finish_meta(0, gi_n, ow_n, k_n);
-    load_w(__builtin_amdgcn_readlane(k_n, 0), w_0);
+    // The first loads are issued in the order the loop issues them (rows of slot u, then the fragments of group u),
+    // pinned against the scheduler: the compiler places one wait count per use for every path into the loop, and a
+    // start that had requested the first group's fragments last would make every block of the loop wait for all but
+    // its last ten loads (the loop's own order lets about thirty stay in flight).
     load_a(gi_n, 0, a_0);
-    load_w(__builtin_amdgcn_readlane(k_n, 1), w_1);
+    __builtin_amdgcn_sched_barrier(0);
+    load_w(__builtin_amdgcn_readlane(k_n, 0), w_0);
+    __builtin_amdgcn_sched_barrier(0);
     load_a(gi_n, 1, a_1);
-    load_w(__builtin_amdgcn_readlane(k_n, 2), w_2);
+    __builtin_amdgcn_sched_barrier(0);
+    load_w(__builtin_amdgcn_readlane(k_n, 1), w_1);
+    __builtin_amdgcn_sched_barrier(0);
     load_a(gi_n, 2, a_2);
+    __builtin_amdgcn_sched_barrier(0);
+    load_w(__builtin_amdgcn_readlane(k_n, 2), w_2);
+    __builtin_amdgcn_sched_barrier(0);
     load_a(gi_n, 3, a_3);
+    __builtin_amdgcn_sched_barrier(0);
 
     for (int g0 = 0; g0 < ngrp; g0 += kBlk) {
         ow_c = ow_n; k_c = k_n;
