@@ -128,9 +128,9 @@ __device__ int block_upper_bound(const int32_t *a, int n, int target, int max_sp
 //   pass 2: one thread per output SLOT reads its group's descriptor, the row at its
 //           rank and the row's table entry, and stores -- consecutive threads store
 //           consecutive slots, so the book is written coalesced.
-// The rule kernels are bound by the number of vector instructions they issue (three
-// waves per SIMD, each instruction four cycles), not by latency: every step above is
-// a handful of instructions per item.
+// A tile's time is the length of its waves' dependent chains (the same with one
+// workgroup per CU as with three): every step above is a handful of instructions per
+// item, batched so that the LDS round trips of several items overlap.
 // ---------------------------------------------------------------------------
 // Lives in dynamic LDS behind the neighbour table, sized by the kernel volume (a 3x3x3 kernel needs 4.5 KB
 // where the largest volume needs 21 KB).
