@@ -102,6 +102,24 @@ def test_random_grids(seed, subm, kernel, stride, padding):
     _check(G.build_case(idx, B, shape, kernel, stride, padding, subm), tile=(2, 2))
 
 
+@pytest.mark.parametrize("B,shape,n,subm,kernel,stride,padding", [
+    (2, [509, 1021, 5], 60000, True, [3, 3, 3], [1, 1, 1], [1, 1, 1]),     # 1.04 M columns, prime line lengths
+    (1, [3, 65537, 9], 40000, True, [3, 3, 3], [1, 1, 1], [1, 1, 1]),      # a line longer than 2^16 columns
+    (5, [127, 129, 33], 50000, False, [3, 3, 3], [2, 2, 2], [1, 1, 1]),
+    (3, [1, 131071, 4], 30000, False, [1, 3, 3], [1, 2, 1], [0, 1, 1]),    # one line per sample, 2^17 - 1 columns
+])
+def test_large_grids_with_odd_line_lengths(B, shape, n, subm, kernel, stride, padding):
+    """A row's column index is split into (batch, S0, S1) with division constants made on the host
+    (multiply-high and shifts): line lengths that are no powers of two, large column indices, the last
+    columns of the last sample occupied.  Pairs against the oracle's, forward and transposed."""
+    rng = np.random.default_rng(shape[1])
+    cells = B * shape[0] * shape[1] * shape[2]
+    lin = rng.choice(cells - 64, size=n, replace=False)
+    lin = np.concatenate([lin, np.arange(cells - 64, cells)])          # the grid's very last cells
+    idx = np.stack(np.unravel_index(lin, (B, *shape)), axis=1).astype(np.int32)
+    _check(G.build_case(idx, B, shape, kernel, stride, padding, subm), tile=(2, 2))
+
+
 def test_deep_axis_more_than_64_bins():
     """S2 = 200 > 64 exercises the multi-pass output-bin masks."""
     rng = np.random.default_rng(3)
