@@ -88,7 +88,18 @@ class Conv3d(Convolution):
                          _triple(padding), _triple(dilation), groups, tile_size, bias, subm, name,
                          indice_key=indice_key, **kwargs)
 
-    def _rules(self, input: SparseConvTensor, out_shape, weight=None):
+    def count_ahead(self, input: SparseConvTensor):
+        """For a strided layer whose rules are not cached: starts counting its output rows on ``input``'s
+        coordinates (RuleBook.count_ahead).  Give the result to ``forward(..., ahead=)`` with a tensor of the
+        same coordinates.  None when there is nothing to do ahead."""
+        if self.subm or input.find_rule(self.indice_key) is not None or not input.z_ptr.is_cuda:
+            return None
+        in_shape = [input.D, input.W, input.H]
+        out_shape = out_spatial(in_shape, self.kernel_size, self.stride, self.padding, self.dilation)
+        return RuleBook.count_ahead(input.z_idx, input.z_ptr, input.B, in_shape, out_shape, self.kernel_size,
+                                    self.stride, self.padding, self.dilation)
+
+    def _rules(self, input: SparseConvTensor, out_shape, weight=None, ahead=None):
         """Rule book of this layer on ``input``, shared through ``rule_cache`` when an
         ``indice_key`` is set (conv.py:159-177).  Returns the cache entry and, when the
         rules had to be generated, the weight packed by the same launch (else None)."""
@@ -103,7 +114,7 @@ class Conv3d(Convolution):
                                        self.padding, self.dilation, weight=weight)
         else:
             book = RuleBook.build(input.z_idx, input.z_ptr, input.B, in_shape, out_shape,
-                                  self.kernel_size, self.stride, self.padding, self.dilation, weight=weight)
+                                  self.kernel_size, self.stride, self.padding, self.dilation, weight=weight, ahead=ahead)
         packed = None
         if weight is not None:
             book, packed = book
@@ -112,17 +123,18 @@ class Conv3d(Convolution):
             input.rule_cache[self.indice_key] = entry
         return entry, packed
 
-    def forward(self, input: SparseConvTensor, epilogue=None) -> SparseConvTensor:
+    def forward(self, input: SparseConvTensor, epilogue=None, ahead=None) -> SparseConvTensor:
         """``epilogue`` = (scale [oC] fp32 or None, shift [oC] fp32 or None, relu): applied to the
         accumulators before the store, inference only (no autograd through it; no reference
-        counterpart)."""
+        counterpart).  ``ahead``: the result of :meth:`count_ahead` on a tensor with this input's
+        coordinates (no reference counterpart either)."""
         assert self.in_channels == input.C, \
             "input channel does not match Expect: {}, got {}".format(self.in_channels, input.C)
         in_shape = [input.D, input.W, input.H]
         out_shape = in_shape if self.subm else out_spatial(in_shape, self.kernel_size, self.stride,
                                                             self.padding, self.dilation)
         weight = self.weight.view(-1, self.in_channels, self.out_channels)
-        (oz_idx, oz_ptr, book, rule_size, tile_grid_shape), packed = self._rules(input, out_shape, weight)
+        (oz_idx, oz_ptr, book, rule_size, tile_grid_shape), packed = self._rules(input, out_shape, weight, ahead)
         self.rule_book = book if isinstance(book, RuleBook) else None
         if epilogue is not None:
             if torch.is_grad_enabled() and (weight.requires_grad or input.feature.requires_grad):

@@ -56,6 +56,12 @@ class Sequential(SphModule):
     ``fuse_eval = False`` switches this off."""
 
     fuse_eval = True
+    # A strided convolution needs its output row count on the host before its rules can be generated.  The
+    # container starts that count as soon as the layer's input coordinates exist -- at the container's input,
+    # or behind the strided layer before it, submanifold layers in between change no coordinates -- so that
+    # the host reads it while the convolutions in between keep the GPU busy (no reference counterpart:
+    # rules.cu:461 waits where the layer runs).  False counts where the layer runs.
+    count_ahead = True
 
     def __init__(self, *args, **kwargs):
         super().__init__()
@@ -109,6 +115,24 @@ class Sequential(SphModule):
         mods = list(self._modules.items())
         only = [m for _, m in mods]
         skip = 0
+        ahead = {}      # index of a strided convolution -> its count on the way
+
+        def start_count(first):
+            """The next strided convolution at or behind module `first` that sees `input`'s coordinates."""
+            if not (self.count_ahead and isinstance(input, SparseConvTensor)):
+                return
+            for j in range(first, len(only)):
+                m = only[j]
+                if is_sparse_conv(m) and not m.subm:
+                    if hasattr(m, "count_ahead"):
+                        h = m.count_ahead(input)
+                        if h is not None:
+                            ahead[j] = h
+                    return
+                if is_sph_module(m) and not is_sparse_conv(m):
+                    return          # a module that may change the coordinates
+
+        start_count(0)
         for i, (name, module) in enumerate(mods):
             if skip:
                 skip -= 1
@@ -117,11 +141,14 @@ class Sequential(SphModule):
                 assert isinstance(input, SparseConvTensor)
                 with torch.autograd.profiler.record_function("sphconv:{}:{}".format(type(module).__name__, name)):
                     skip, bn, relu = self._fusable_tail(only, i)
+                    kw = {"ahead": ahead.pop(i)} if i in ahead else {}
                     if skip:
                         scale, shift = _bn_affine(bn) if bn is not None else (None, None)
-                        input = module(input, epilogue=(scale, shift, relu))
+                        input = module(input, epilogue=(scale, shift, relu), **kw)
                     else:
-                        input = module(input)
+                        input = module(input, **kw)
+                    if is_sparse_conv(module) and not module.subm:
+                        start_count(i + 1)      # new coordinates: the next strided layer can start counting
             elif isinstance(input, SparseConvTensor):
                 input.feature = module(input.feature)
             else:

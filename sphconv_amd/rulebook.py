@@ -203,12 +203,12 @@ class RuleBook:
         return rb, packed
 
     @classmethod
-    def build(cls, z_idx, z_ptr, batch, in_shape, out_shape, kernel, stride, padding,
-              dilation=(1, 1, 1), weight=None):
-        """Strided rules (replaces get_rules, rules.cu:405-486): output coordinates
-        (oz_ptr inclusive scan, oz_idx ascending per column) and pairs.  One wait for the
-        output row count, as in the reference (rules.cu:461): the count kernel writes it to pinned
-        host memory, so the wait is a stream synchronisation and no copy."""
+    def count_ahead(cls, z_idx, z_ptr, batch, in_shape, out_shape, kernel, stride, padding, dilation=(1, 1, 1)):
+        """First half of :meth:`build`, to be enqueued as soon as a strided layer's INPUT coordinates exist:
+        the output rows per column are counted and scanned, the row count goes to pinned host memory, and an
+        event marks the place in the stream.  Pass the returned object to ``build(..., ahead=)`` when the layer
+        itself is reached: whatever the caller has enqueued in between (the convolutions of the layers before)
+        keeps the GPU busy while the host reads the count, instead of the GPU waiting for the host."""
         _check_index_tensors(z_idx, z_ptr, batch, in_shape)
         lib = L.lib()
         dev = z_ptr.device
@@ -219,21 +219,64 @@ class RuleBook:
         if nints < 0:
             L.check(nints)
         oz_ptr = torch.empty((int(batch), int(out_shape[0]), int(out_shape[1])), dtype=torch.int32, device=dev)
-        scratch, total = _outcoords_workspace(dev, nints)
+        # scratch and the pinned word are this call's own: other strided layers may be generated before build()
+        scratch = torch.empty(max(nints + (nints & 1), 2), dtype=torch.int32, device=dev)
+        total = _pinned_word()
+        stream = torch.cuda.current_stream(dev)
+        L.check(lib.sph_outcoords_count(L.ptr(z_idx), L.ptr(z_ptr), int(z_idx.shape[0]), C.byref(g), L.ptr(oz_ptr),
+                                        L.ptr(scratch), total.data_ptr(), stream.cuda_stream))
+        event = torch.cuda.Event()
+        event.record(stream)
+        key = (z_idx.data_ptr(), z_ptr.data_ptr(), int(batch), tuple(int(v) for v in in_shape),
+               tuple(int(v) for v in out_shape), tuple(int(v) for v in kernel), tuple(int(v) for v in stride),
+               tuple(int(v) for v in padding), tuple(int(v) for v in dilation))
+        return _CountAhead(key, oz_ptr, scratch, total, event, stream.cuda_stream)
+
+    @classmethod
+    def build(cls, z_idx, z_ptr, batch, in_shape, out_shape, kernel, stride, padding,
+              dilation=(1, 1, 1), weight=None, ahead=None):
+        """Strided rules (replaces get_rules, rules.cu:405-486): output coordinates
+        (oz_ptr inclusive scan, oz_idx ascending per column) and pairs.  One wait for the
+        output row count, as in the reference (rules.cu:461): the count kernel writes it to pinned
+        host memory, so the wait is a stream synchronisation and no copy.  ``ahead``: what
+        :meth:`count_ahead` returned for the same arguments on the same stream; the wait is then for its
+        event only."""
+        _check_index_tensors(z_idx, z_ptr, batch, in_shape)
+        lib = L.lib()
+        dev = z_ptr.device
+        g = L.make_geom(batch, in_shape, out_shape, kernel, stride, padding, dilation)
+        if min(int(v) for v in out_shape) <= 0:
+            raise L.SphconvError("empty output grid %s" % (list(out_shape),))
         n_in = int(z_idx.shape[0])
         stream = torch.cuda.current_stream(dev)
-        try:
-            # one launch: counts, their scan into oz_ptr, and the row count written straight to pinned host memory
-            L.check(lib.sph_outcoords_count(L.ptr(z_idx), L.ptr(z_ptr), n_in, C.byref(g), L.ptr(oz_ptr),
-                                            L.ptr(scratch), total.data_ptr(), stream.cuda_stream))
-            stream.synchronize()             # the one wait of a strided layer (the reference's is rules.cu:461)
-        except Exception:
-            _WORKSPACES.pop(_workspace_key(dev), None)   # whatever failed, the next call starts from fresh buffers
-            raise
+        if ahead is not None:
+            key = (z_idx.data_ptr(), z_ptr.data_ptr(), int(batch), tuple(int(v) for v in in_shape),
+                   tuple(int(v) for v in out_shape), tuple(int(v) for v in kernel), tuple(int(v) for v in stride),
+                   tuple(int(v) for v in padding), tuple(int(v) for v in dilation))
+            if ahead.key != key or ahead.stream != stream.cuda_stream:
+                raise L.SphconvError("count_ahead() was called for another layer, tensor or stream")
+            oz_ptr, scratch, total = ahead.oz_ptr, ahead.scratch, ahead.total
+            ahead.event.synchronize()
+        else:
+            nints = lib.sph_outcoords_scratch_ints(C.byref(g))
+            if nints < 0:
+                L.check(nints)
+            oz_ptr = torch.empty((int(batch), int(out_shape[0]), int(out_shape[1])), dtype=torch.int32, device=dev)
+            scratch, total = _outcoords_workspace(dev, nints)
+            try:
+                # one launch: counts, their scan into oz_ptr, and the row count written straight to pinned host memory
+                L.check(lib.sph_outcoords_count(L.ptr(z_idx), L.ptr(z_ptr), n_in, C.byref(g), L.ptr(oz_ptr),
+                                                L.ptr(scratch), total.data_ptr(), stream.cuda_stream))
+                stream.synchronize()             # the one wait of a strided layer (the reference's is rules.cu:461)
+            except Exception:
+                _WORKSPACES.pop(_workspace_key(dev), None)   # whatever failed, the next call starts from fresh buffers
+                raise
         out_rows = int(total[0])
         oz_idx = torch.empty(out_rows, dtype=torch.int32, device=dev)
         L.check(lib.sph_outcoords_fill(L.ptr(z_idx), L.ptr(z_ptr), n_in, C.byref(g), L.ptr(scratch),
                                        L.ptr(oz_ptr), L.ptr(oz_idx), out_rows, L.stream()))
+        if ahead is not None:
+            _release_pinned_word(total)
         rb = cls(z_idx, z_ptr, oz_idx, oz_ptr, batch, in_shape, out_shape, kernel, stride, padding,
                  dilation, False)
         if weight is None:
@@ -357,6 +400,27 @@ def _outcoords_workspace(dev, nints: int):
         ws = (scratch, total)
         _WORKSPACES[key] = ws
     return ws
+
+
+class _CountAhead:
+    """Output-row counts of a strided layer on their way (RuleBook.count_ahead)."""
+
+    def __init__(self, key, oz_ptr, scratch, total, event, stream):
+        self.key, self.oz_ptr, self.scratch, self.total, self.event, self.stream = key, oz_ptr, scratch, total, event, stream
+
+
+# Pinned host words that receive row counts; handed out one per count in flight and taken back when read
+# (pinning memory costs a system call, so they are never freed).
+_PINNED_WORDS = []
+
+
+def _pinned_word():
+    return _PINNED_WORDS.pop() if _PINNED_WORDS else torch.zeros(1, dtype=torch.int32).pin_memory()
+
+
+def _release_pinned_word(word):
+    if len(_PINNED_WORDS) < 64:
+        _PINNED_WORDS.append(word)
 
 
 def _check_index_tensors(z_idx, z_ptr, batch, shape):

@@ -232,6 +232,51 @@ def test_fused_eval_tail_equals_separate_modules():
     assert torch.equal(y3.feature.detach(), plain.feature)
 
 
+def test_strided_row_counts_started_ahead_change_nothing():
+    """A container starts a strided layer's output-row count when the layer's input coordinates exist and
+    hands it to the layer when it runs: same coordinates, same features, bit for bit, as counting where the
+    layer runs -- under no_grad (fused tails) and with autograd; and the two halves used directly."""
+    from sphconv_amd import _lib as L
+    from sphconv_amd.rulebook import RuleBook
+    from sphconv_amd.synth import encoder_stack
+    B, shape = 3, [16, 40, 16]
+    idx, feat = _inputs(9, B, shape, 16, p=0.15)
+    net = encoder_stack(16, (16, 32, 32), seed=2).to(G.DEV).half()
+    assert net.count_ahead
+    outs = {}
+    for ahead in (True, False):
+        net.count_ahead = ahead
+        with torch.no_grad():
+            y = net(sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx)))
+        outs[ahead] = y
+        f = G.t(feat).half().requires_grad_(True)
+        yg = net(sphconv.SparseConvTensor(f, shape, B, indices=G.t(idx)))
+        yg.feature.float().square().sum().backward()
+        outs[ahead, "grad"] = (yg.feature.detach(), f.grad.clone(), [p.grad.clone() for p in net.parameters() if p.grad is not None])
+        net.zero_grad()
+    net.count_ahead = True
+    a, b = outs[True], outs[False]
+    assert a.feature.shape[0] > 0 and float(a.feature.float().abs().mean()) > 1e-3
+    assert torch.equal(a.z_idx, b.z_idx) and torch.equal(a.z_ptr, b.z_ptr) and torch.equal(a.feature, b.feature)
+    (ya, ga, pa), (yb, gb, pb) = outs[True, "grad"], outs[False, "grad"]
+    assert torch.equal(ya, yb) and torch.equal(ga, gb) and len(pa) == len(pb) > 0
+    assert all(torch.equal(u, v) for u, v in zip(pa, pb))
+    # the two halves by hand, with other work (another strided layer's rules) enqueued in between
+    x = sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx))
+    args = (x.z_idx, x.z_ptr, B, shape, [8, 20, 8], [3, 3, 3], [2, 2, 2], [1, 1, 1])
+    h = RuleBook.count_ahead(*args)
+    other = RuleBook.build(x.z_idx, x.z_ptr, B, shape, [14, 38, 14], [3, 3, 3], [1, 1, 1], [0, 0, 0])
+    late = RuleBook.build(*args, ahead=h)
+    plain = RuleBook.build(*args)
+    assert other.out_rows > 0 and late.out_rows == plain.out_rows > 0
+    assert torch.equal(late.oz_idx, plain.oz_idx) and torch.equal(late.oz_ptr, plain.oz_ptr)
+    assert np.array_equal(G.book_triples(late.fwd), G.book_triples(plain.fwd))
+    # a count started for one layer is refused by another
+    h2 = RuleBook.count_ahead(*args)
+    with pytest.raises(L.SphconvError, match="another layer"):
+        RuleBook.build(x.z_idx, x.z_ptr, B, shape, [14, 38, 14], [3, 3, 3], [1, 1, 1], [0, 0, 0], ahead=h2)
+
+
 def test_config4_encoder_full_size_layer_by_layer():
     """BASELINE configuration 4 (batch 4, grid 64x2048x64, four stages of two submanifold and one
     strided convolution, BatchNorm + ReLU fused, fp16): every layer's output against the C oracle
