@@ -2,24 +2,29 @@
 """Benchmark of the sparse-convolution hot path on one MI355X.
 
 One step = rule generation + forward of one 3x3x3 submanifold convolution
-64->64, fp16 storage / fp32 accumulate (two kernel launches: the rule kernel, which
-also carries the per-step weight packing as extra workgroups, and the convolution),
-on one synthetic LiDAR-like scan
+64->64, fp16 storage / fp32 accumulate, on one synthetic LiDAR-like scan
 (config-2 generator: 64 x 2048 x 64 range grid, ~95-120k active voxels), with
-the scan's index arrays, features and weights already resident in HBM.
+the scan (index arrays, the rows' columns, features) and the layer's weight (in the
+kernel's fragment order, as a serving pipeline keeps it) already resident in HBM.
+A scan of up to 1024 tiles takes ONE launch (sph_rules_conv: every workgroup makes
+its tile's rules in LDS and convolves them at once), a larger one two.
 
 The timed steps are dealt to a few HIP streams (--streams, default 3): every step redoes all
-of its work into per-stream buffers, but the rule kernel of one scan can run beside the
-convolution of another.  `one_stream_ms_per_step` is the same step with one scan at a time.
-The steps walk through --scans resident copies of the scan (more memory than the last-level
-cache holds); the timed loop of --steps steps is repeated --repeats times and the median counts,
-after the per-kernel section has settled the device.
+of its work into per-stream buffers, the kernels of one scan run beside those of another.
+`one_stream_ms_per_step` is the same step with one scan at a time through the extension's
+Python API.  The steps walk through --scans resident copies of the scan (more memory than the
+last-level cache holds); the timed loop of --steps steps is repeated --repeats times and the
+median counts, after the per-kernel section has settled the device.  `ms_per_step` is device
+time (HIP events on the streams: last end - first start), `host_ms_per_step` the host's clock
+around the same region between device synchronisations.
 
 Prints ONE JSON line:  value = active voxels / second over the timed steps,
-plus `rulegen_ms_per_scan`, a `roofline` object for the dominant kernel (live
-HIP-event timing of that kernel alone), an `at_120k` object (the same step on a scan of the
-size BASELINE's metric names) and a `cpu_baseline` object (the CPU restatement of the reference
-algorithm under oracle/, timed on this host).
+plus `rulegen_ms_per_scan`, `roofline` objects (live HIP-event timing of each kernel alone:
+the step's own kernel, and the rule kernel and the convolution kernel of the two-launch path),
+`mfma` (useful and executed matrix flops against the fp16 peak), an `at_120k` object (the same
+step on a scan of the size BASELINE's metric names) and a `cpu_baseline` object (the CPU
+restatement of the reference algorithm under oracle/, timed on this host, with the dense
+conv3d of configuration 1 beside it as a sanity line).
 """
 import argparse
 import json
@@ -31,6 +36,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
 def parse():
@@ -114,17 +120,60 @@ def cpu_baseline(d, ic, oc, budget_s, seed):
         t2 = time.perf_counter()
         return t1 - t0, t2 - t1, dropped
 
-    one()  # warm-up (page faults of the 1.8 GB padded rule tensor)
+    for _ in range(3):  # warm-ups (the first also takes the page faults of the 1.8 GB padded rule tensor)
+        one()
     times, t_start = [], time.perf_counter()
-    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 50):
+    while len(times) < 10 or (time.perf_counter() - t_start < budget_s and len(times) < 50):
         times.append(one())
     rg = sorted(t[0] for t in times)[len(times) // 2]
     fw = sorted(t[1] for t in times)[len(times) // 2]
     return {"value": n / (rg + fw), "unit": "voxels/s", "cores": cores, "kind": "port",
-            "sample": "%d scans of the same %d-voxel scan, median; rulegen %.1f ms + forward %.1f ms, "
+            "sample": "3 warm-ups, then %d scans of the same %d-voxel scan, median; rulegen %.1f ms + forward %.1f ms, "
                       "fp32, tile 2x2, tile_n_max %d, dropped pairs %d"
                       % (len(times), n, rg * 1e3, fw * 1e3, n_max, times[0][2]),
-            "rulegen_ms": rg * 1e3, "forward_ms": fw * 1e3}
+            "rulegen_ms": rg * 1e3, "forward_ms": fw * 1e3,
+            "config1_sanity": config1_sanity(cores, seed)}
+
+
+def config1_sanity(cores, seed):
+    """Configuration 1 (64 x 512 x 32 grid, 16 -> 16 fp32) on the host: the CPU restatement (rules + forward) and,
+    beside it, the dense alternative torch.nn.functional.conv3d over the whole grid.  Not the baseline."""
+    import numpy as np
+    import torch
+    from oracle import oracle as O
+    from sphconv_amd.synth import make_config
+    d = make_config(1, seed=seed)
+    shape, B = d["spatial_shape"], d["batch"]
+    n = int(d["z_idx"].shape[0])
+    rng = np.random.default_rng(seed)
+    feat = rng.standard_normal((n, 16)).astype(np.float32)
+    w = (rng.standard_normal((27, 16, 16)) / np.sqrt(27 * 16)).astype(np.float32)
+
+    def sparse():
+        _, _, rules, rule_size, _ = O.get_rules_subm(d["z_idx"], d["z_ptr"], B, shape, shape, [3, 3, 3], [1, 1, 1],
+                                                     [1, 1, 1], canonical=False)
+        return O.rule_conv(feat, w, rules, rule_size, n)
+
+    idx = torch.tensor(d["indices"].astype(np.int64))
+    dense = torch.zeros((B, 16, *shape))
+    dense[idx[:, 0], :, idx[:, 1], idx[:, 2], idx[:, 3]] = torch.tensor(feat)
+    wd = torch.tensor(w).reshape(3, 3, 3, 16, 16).permute(4, 3, 0, 1, 2).contiguous()
+    torch.set_num_threads(cores)
+
+    def timed(fn, reps):
+        for _ in range(3):
+            fn()
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return sorted(ts)[len(ts) // 2] * 1e3
+
+    return {"voxels": n, "cpu_restatement_ms": timed(sparse, 10),
+            "dense_conv3d_ms": timed(lambda: torch.nn.functional.conv3d(dense, wd, padding=1), 5),
+            "note": "3 warm-ups, median; dense = torch conv3d over all %d cells, fp32, %d threads"
+                    % (B * shape[0] * shape[1] * shape[2], cores)}
 
 
 def encoder_stack_ms(torch, seed, iters):
@@ -309,11 +358,11 @@ def configs_ms(torch, seed, iters):
 
 
 def kernel_sources_digest():
-    """sha256 over the sources of the two kernels whose HBM traffic is on record (what a counter run was
+    """sha256 over the sources of the kernels whose HBM traffic is on record (what a counter run was
     taken on): the recorded traffic is only reported while these files are what it was measured on."""
     import hashlib
     h = hashlib.sha256()
-    for name in ("conv.hip", "rules.hip", "common.h", "pack.h"):
+    for name in ("conv.hip", "rules.hip", "fused.hip", "conv_wave.h", "rules_tile.h", "tile_consts.h", "common.h", "pack.h"):
         with open(os.path.join(ROOT, "sphconv_amd", "csrc", name), "rb") as f:
             h.update(f.read())
     return h.hexdigest()
@@ -373,10 +422,11 @@ def record_traffic(fetch_csv, write_csv, seed, voxels):
     kernels = []
     for n in sizes:
         blocks = ((n + 127) // 128 + 7) // 8 * 8        # tiles, rounded up to whole rounds over the 8 XCDs
+        tiles = (n + 127) // 128
         wanted = {"conv": ("conv_wave_kernel", lambda g: g == blocks * 64),
-                  # the step's launch: one workgroup of 256 threads per tile, then the ones that pack the weight
-                  # (the per-kernel section also launches it without them)
-                  "rules": ("build_book_kernel<false>", lambda g: blocks * 256 < g <= (blocks + 512) * 256)}
+                  "rules": ("build_book_kernel<false>", lambda g: g == blocks * 256),
+                  # one launch: workgroups of 256 threads up to 768 tiles, of 128 beyond
+                  "rules_conv": ("rules_conv_kernel", lambda g: g == blocks * (256 if tiles <= 768 else 128))}
         for key, (pat, grid_ok) in wanted.items():
             def mean(per):
                 vals = [v for (name, g), vs in per.items() if pat in name and grid_ok(g) for v in vs]
@@ -400,11 +450,12 @@ def record_traffic(fetch_csv, write_csv, seed, voxels):
 
 
 class Workload:
-    """One scan size of the benchmark: `copies` device-resident copies of the scan (index arrays and
-    features in separate allocations, so that the timed steps walk through more memory than the 256 MB
-    last-level cache holds), and the timings of the step on it."""
+    """One scan size of the benchmark: `copies` device-resident copies of the scan (index arrays, the rows'
+    columns and features in separate allocations, so that the timed steps walk through more memory than the
+    256 MB last-level cache holds), and the timings of the step on it."""
 
     def __init__(self, torch, d, ic, oc, w, copies, seed):
+        from sphconv_amd.rulebook import row_columns
         self.torch = torch
         self.d, self.ic, self.oc, self.w = d, ic, oc, w
         self.shape, self.B = d["spatial_shape"], d["batch"]
@@ -415,84 +466,129 @@ class Workload:
         self.scans = []
         for _ in range(copies):
             feat = torch.randn((self.n, ic), device=dev, generator=gen).half()
-            self.scans.append((feat, zi.to(dev).clone(), zp.to(dev).clone()))
-        self.footprint = copies * (self.n * ic * 2 + self.n * 4 + zp.numel() * 4)
+            z_idx, z_ptr = zi.to(dev).clone(), zp.to(dev).clone()
+            # the rows' columns: part of the tensor, as init_tensor and the output-coordinate kernels leave it
+            self.scans.append((feat, z_idx, z_ptr, row_columns(z_ptr, self.n)))
+        self.footprint = copies * (self.n * ic * 2 + self.n * 8 + zp.numel() * 4)
 
     def step(self, i):
-        """rule generation (the weight is put in MFMA fragment order by extra workgroups of the same launch,
-        every step) + forward, on copy i of the scan."""
+        """Rule generation + forward on copy i of the scan through the extension's Python API: a rule book that
+        is not built yet, and rule_conv, which makes its pairs in the launch that convolves them (the weight's
+        fragment-ordered copy is kept with the weight, as for a module in eval mode)."""
         from sphconv_amd import sphconv_cuda as ext
         from sphconv_amd.rulebook import RuleBook
-        feat, z_idx, z_ptr = self.scans[i % len(self.scans)]
-        book, packed = RuleBook.build_subm(z_idx, z_ptr, self.B, self.shape, [3, 3, 3], weight=self.w)
-        return book, ext.rule_conv(feat, self.w, book, None, self.n, packed=packed)
+        feat, z_idx, z_ptr, cols = self.scans[i % len(self.scans)]
+        book = RuleBook.build_subm(z_idx, z_ptr, self.B, self.shape, [3, 3, 3], row_cols=cols, lazy=True)
+        book.keep = False
+        return book, ext.rule_conv(feat, self.w, book, None, self.n, cache_packed=True)
 
     def time_one_stream(self, steps, warmup, repeats):
         torch = self.torch
-        for i in range(warmup):
-            self.step(i)
-        torch.cuda.synchronize()
-        times = []
-        for r in range(repeats):
-            t0 = time.perf_counter()
-            for i in range(steps):
-                self.step(r * steps + i)
+        with torch.no_grad():
+            for i in range(warmup):
+                self.step(i)
             torch.cuda.synchronize()
-            times.append((time.perf_counter() - t0) / steps * 1e3)
-        return sorted(times)[len(times) // 2], times
+            times, dev_times = [], []
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            for r in range(repeats):
+                t0 = time.perf_counter()
+                e0.record()
+                for i in range(steps):
+                    self.step(r * steps + i)
+                e1.record()
+                torch.cuda.synchronize()
+                times.append((time.perf_counter() - t0) / steps * 1e3)
+                dev_times.append(e0.elapsed_time(e1) / steps)
+        return sorted(dev_times)[len(dev_times) // 2], sorted(times)[len(times) // 2], dev_times
 
-    def time_pipelined(self, steps, warmup, repeats, streams):
-        """The same two launches per scan, scans dealt to a few HIP streams so that the rule kernel of one scan
-        runs beside the convolution of another (a 100k-voxel scan fills neither kernel's grid); buffers are
-        allocated once per stream slot, every step redoes all the work."""
+    def time_pipelined(self, steps, warmup, repeats, streams, fused=True):
+        """The same step per scan, scans dealt to a few HIP streams so that the kernels of one scan run beside
+        those of another (a 100k-voxel scan does not fill the chip); buffers are allocated once per stream slot,
+        every step redoes all the work.  Device time of a repeat: from the first start to the last end over the
+        streams (an event at the head of every stream's share of the steps and one at its tail, against one
+        reference event); host time: the host's clock between the device synchronisations around it."""
         torch = self.torch
         from sphconv_amd.pipeline import ScanPipeline
-        pipe = ScanPipeline(self.w, self.B, self.shape, max_voxels=self.n, streams=streams)
+        pipe = ScanPipeline(self.w, self.B, self.shape, max_voxels=self.n, streams=streams, fused=fused)
+
+        def submit(k):
+            feat, z_idx, z_ptr, cols = self.scans[k % len(self.scans)]
+            return pipe.submit(feat, z_idx, z_ptr, wait_inputs=False, row_cols=cols)   # inputs are resident and complete
+
         for i in range(warmup):
-            pipe.submit(*self.scans[i % len(self.scans)], wait_inputs=False)
+            submit(i)
         pipe.synchronize()
         torch.cuda.synchronize()
-        times = []
+        ns = pipe.streams
+        ref = torch.cuda.Event(enable_timing=True)
+        heads = [torch.cuda.Event(enable_timing=True) for _ in range(ns)]
+        tails = [torch.cuda.Event(enable_timing=True) for _ in range(ns)]
+        times, dev_times = [], []
         last = None
         for r in range(repeats):
             t0 = time.perf_counter()
+            ref.record()
             for i in range(steps):
+                slot = pipe.next_slot()
+                if i < ns:
+                    heads[slot].record(pipe.stream_of(slot))
                 k = (r * steps + i) % len(self.scans)
-                last = (pipe.submit(*self.scans[k], wait_inputs=False), k)   # inputs are resident and complete
+                last = (submit(k), k)
+                if i >= steps - ns:
+                    tails[slot].record(pipe.stream_of(slot))
             torch.cuda.synchronize()      # every stream of the device (one wait, not one per stream)
             times.append((time.perf_counter() - t0) / steps * 1e3)
+            used = min(ns, steps)
+            slots = [(pipe.next_slot() - 1 - q) % ns for q in range(used)]
+            start = min(ref.elapsed_time(heads[q]) for q in slots)
+            end = max(ref.elapsed_time(tails[q]) for q in slots)
+            dev_times.append((end - start) / steps)
         (out_p, _slot), k = last
         _, out = self.step(k)
-        assert torch.equal(out_p, out)
-        return sorted(times)[len(times) // 2], times
+        err = float((out_p.float() - out.float()).abs().max())
+        assert err <= 1e-2 * max(1.0, float(out.float().abs().max())), err
+        return sorted(dev_times)[len(dev_times) // 2], sorted(times)[len(times) // 2], dev_times
 
     def time_kernels(self, iters, backward=False, rng=None):
         """Each kernel alone: HIP events on the launch stream around `iters` back-to-back launches."""
         import ctypes as C
         from sphconv_amd import _lib as L
         from sphconv_amd import sphconv_cuda as ext
+        from sphconv_amd.rulebook import RuleBook, _Buffers
         torch = self.torch
         lib = L.lib()
-        feat, z_idx, z_ptr = self.scans[0]
+        feat, z_idx, z_ptr, cols = self.scans[0]
         n, ic, oc, w = self.n, self.ic, self.oc, self.w
-        book, out = self.step(0)
+        book = RuleBook.build_subm(z_idx, z_ptr, self.B, self.shape, [3, 3, 3], row_cols=cols)
+        out = ext.rule_conv(feat, w, book, None, n)
         self.pairs = book.num_pairs()
         g = book.geom()
         bk = book.fwd.struct()
         stream = L.stream()
+        zi, zp = z_idx.data_ptr(), z_ptr.data_ptr()
         res = {}
-        res["rulegen_ms"] = event_ms(lambda: lib.sph_rules_build(z_idx.data_ptr(), z_ptr.data_ptr(), n, z_idx.data_ptr(),
-                                                                 z_ptr.data_ptr(), n, C.byref(g), 0, C.byref(bk), stream),
-                                     iters, torch)
+        res["rulegen_ms"] = event_ms(lambda: lib.sph_rules_build(zi, zp, n, zi, zp, n, C.byref(g), 0, C.byref(bk),
+                                                                 cols.data_ptr(), stream), iters, torch)
+        res["rulegen_without_columns_ms"] = event_ms(lambda: lib.sph_rules_build(zi, zp, n, zi, zp, n, C.byref(g), 0,
+                                                                                 C.byref(bk), None, stream), iters, torch)
         packed = ext._packed_weight(w, False)
         out_buf = torch.empty((n, oc), dtype=torch.float16, device=w.device)
         epi = L.Epilogue(None, None, 0)
         res["conv_forward_ms"] = event_ms(lambda: lib.sph_conv_apply(L.F16, feat.data_ptr(), n, ic, packed.data_ptr(), oc,
                                                                      C.byref(bk), C.byref(epi), out_buf.data_ptr(), stream),
                                           iters, torch)
+        assert torch.equal(out_buf, out)
         res["weight_pack_ms"] = event_ms(lambda: lib.sph_weight_pack(L.F16, w.data_ptr(), 27, ic, oc, ic * oc, oc, 1,
                                                                      packed.data_ptr(), stream), iters, torch)
-        assert torch.equal(out_buf, out)
+        scratch_book = _Buffers(n, 27, w.device)
+        sb = scratch_book.struct()
+        one = lambda: lib.sph_rules_conv(zi, zp, n, zi, zp, n, C.byref(g), C.byref(sb), 0, cols.data_ptr(), L.F16,
+                                         feat.data_ptr(), ic, packed.data_ptr(), oc, C.byref(epi), out_buf.data_ptr(), stream)
+        self.one_launch = one() == 0
+        if self.one_launch:
+            res["rules_conv_one_launch_ms"] = event_ms(one, iters, torch)
+            err = float((out_buf.float() - out.float()).abs().max())
+            assert err <= 1e-2 * max(1.0, float(out.float().abs().max())), err
         if backward:
             d_out = torch.randn((n, oc), device=w.device).half()
             w_t = w.permute(0, 2, 1).contiguous()
@@ -502,24 +598,48 @@ class Workload:
             res["wgrad_ms"] = event_ms(lambda: ext.rule_conv_d_weight(feat, d_out, book, None), iters, torch)
         e, P = 2, self.pairs
         nt = book.fwd.ntiles
+        self.flops = 2.0 * P * ic * oc
+        self.ntiles = nt
+        self.executed_groups = int(book.fwd.tile_ngrp[:nt].sum())
         self.conv_bytes = n * ic * e + n * oc * e + 27 * ic * oc * e + 8 * P
-        self.rule_bytes = 4 * z_ptr.numel() + 4 * n + 8 * P + nt * (4 + 2 * 28)
+        self.rule_bytes = 4 * z_ptr.numel() + 4 * n + 4 * n + 8 * P + nt * (4 + 2 * 28)   # + the rows' columns
+        # one launch: the scan and the weight in, the output rows out; the pairs never leave the chip
+        self.fused_bytes = 4 * z_ptr.numel() + 4 * n + 4 * n + n * ic * e + n * oc * e + 27 * ic * oc * e
         res["rulegen_GBps"] = self.rule_bytes / (res["rulegen_ms"] * 1e-3) / 1e9
         res["conv_GBps"] = self.conv_bytes / (res["conv_forward_ms"] * 1e-3) / 1e9
-        res["conv_TFLOPs"] = 2.0 * P * ic * oc / (res["conv_forward_ms"] * 1e-3) / 1e12
+        res["conv_TFLOPs"] = self.flops / (res["conv_forward_ms"] * 1e-3) / 1e12
         return res
 
-    def roofline(self, kern, seed):
-        """For the kernel that lasts longest: algorithmic bytes per launch / its average duration, against the
-        HBM peak."""
-        if kern["conv_forward_ms"] >= kern["rulegen_ms"]:
-            dom = ("conv_wave_kernel<f16,2,4,false>", self.conv_bytes, kern["conv_forward_ms"], "conv")
-        else:
-            dom = ("build_book_kernel<false>", self.rule_bytes, kern["rulegen_ms"], "rules")
-        achieved = dom[1] / (dom[2] * 1e-3) / 1e9
+    def _roofline(self, kernel, key, nbytes, ms, seed):
+        achieved = nbytes / (ms * 1e-3) / 1e9
         return {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic(dom[3], self.n, seed),
-                "kernel": dom[0], "algorithmic_bytes": dom[1], "kernel_ms": dom[2]}
+                "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic(key, self.n, seed),
+                "kernel": kernel, "algorithmic_bytes": nbytes, "kernel_ms": ms}
+
+    def rooflines(self, kern, seed):
+        """(the step's dominant kernel, the rule kernel, the convolution kernel): algorithmic bytes per launch over
+        the kernel's average duration, against the HBM peak."""
+        rules = self._roofline("build_book_kernel<false>", "rules", self.rule_bytes, kern["rulegen_ms"], seed)
+        conv = self._roofline("conv_wave_kernel<f16,2,4,false>", "conv", self.conv_bytes, kern["conv_forward_ms"], seed)
+        if self.one_launch:
+            name = "rules_conv_kernel<f16,2,4,false,%d>" % (256 if self.ntiles <= 768 else 128)
+            main = self._roofline(name, "rules_conv", self.fused_bytes, kern["rules_conv_one_launch_ms"], seed)
+        else:
+            main = conv if kern["conv_forward_ms"] >= kern["rulegen_ms"] else rules
+        return main, rules, conv
+
+    def mfma(self, kern):
+        """Matrix-unit figures of the convolution: useful flops (2 x pairs x iC x oC) over the kernel's duration
+        against the fp16 MFMA peak, and what the kernel executes for them (whole groups of 16 pairs: the padding
+        slots of a group are multiplied too)."""
+        ms = kern.get("rules_conv_one_launch_ms", kern["conv_forward_ms"]) if self.one_launch else kern["conv_forward_ms"]
+        groups = self.executed_groups
+        executed = 2.0 * groups * 16 * self.ic * self.oc
+        return {"useful_flops": self.flops, "executed_flops": executed, "executed_over_useful": executed / self.flops,
+                "conv_kernel_TFLOPs": self.flops / (kern["conv_forward_ms"] * 1e-3) / 1e12,
+                "conv_kernel_frac_of_peak": self.flops / (kern["conv_forward_ms"] * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
+                "step_kernel_frac_of_peak": self.flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
+                "peak_TFLOPs": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s"}
 
 
 def main():
@@ -559,39 +679,52 @@ def main():
         # timed run (--steps 20) reads the same as a long one
         iters = max(100, min(args.steps, 200))
         kern = wl.time_kernels(iters, backward=args.backward, rng=rng)
-        one_ms, one_all = wl.time_one_stream(args.steps, max(args.warmup, 20), args.repeats)
-        ms, ms_all = wl.time_pipelined(args.steps, max(args.warmup, 20), args.repeats, args.streams)
-        return wl, kern, one_ms, ms, {"one_stream_ms": one_all, "pipelined_ms": ms_all}
+        one_dev, one_host, one_all = wl.time_one_stream(args.steps, max(args.warmup, 20), args.repeats)
+        ms, host_ms, ms_all = wl.time_pipelined(args.steps, max(args.warmup, 20), args.repeats, args.streams)
+        two = wl.time_pipelined(args.steps, max(args.warmup, 20), args.repeats, args.streams, fused=False)
+        return wl, kern, {"ms": ms, "host_ms": host_ms, "one_stream_ms": one_dev, "one_stream_host_ms": one_host,
+                          "two_launch_ms": two[0], "two_launch_host_ms": two[1],
+                          "repeats": {"one_stream_ms": one_all, "pipelined_ms": ms_all}}
 
-    wl, kern, one_stream_ms, ms_per_step, repeats = measure(d)
+    def report(wl, kern, t):
+        main_roof, rules_roof, conv_roof = wl.rooflines(kern, args.seed)
+        return {"ms_per_step": t["ms"], "host_ms_per_step": t["host_ms"],
+                "one_stream_ms_per_step": t["one_stream_ms"], "one_stream_host_ms_per_step": t["one_stream_host_ms"],
+                "two_launch_ms_per_step": t["two_launch_ms"], "two_launch_host_ms_per_step": t["two_launch_host_ms"],
+                "launches_per_step": 1 if wl.one_launch else 2,
+                "rulegen_ms_per_scan": kern["rulegen_ms"], "kernels": kern, "roofline": main_roof,
+                "roofline_rules": rules_roof, "roofline_conv": conv_roof, "mfma": wl.mfma(kern), "repeats": t["repeats"]}
+
+    wl, kern, t = measure(d)
     n, P = wl.n, wl.pairs
+    rep = report(wl, kern, t)
     result = {
         "metric": "active voxels/sec, 3x3x3 subm conv 64->64 fp16 (rulegen + forward); rulegen ms/scan",
-        "value": n / (ms_per_step * 1e-3), "unit": "voxels/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "value": n / (rep["ms_per_step"] * 1e-3), "unit": "voxels/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": rep["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "config-2 generator (G2, seed %d): grid 64x2048x64, batch 1, %d active voxels, "
-                               "%d pairs; subm 3x3x3 64->64, fp16 storage / fp32 accumulate; the timed steps walk "
-                               "through %d resident copies of the scan (%d MB) on %d HIP streams; ms_per_step is the "
-                               "median of %d repeats of `steps` steps"
-                               % (args.seed, n, P, args.scans, wl.footprint >> 20, args.streams, args.repeats),
+                               "%d pairs; subm 3x3x3 64->64, fp16 storage / fp32 accumulate; rules + forward in %d "
+                               "launch(es) per scan; the timed steps walk through %d resident copies of the scan "
+                               "(%d MB) on %d HIP streams; ms_per_step is device time (HIP events on the streams), "
+                               "the median of %d repeats of `steps` steps"
+                               % (args.seed, n, P, rep["launches_per_step"], args.scans, wl.footprint >> 20, args.streams,
+                                  args.repeats),
                    "grid": wl.shape, "batch": wl.B, "voxels": n, "pairs": P, "channels": [ic, oc]},
-        "rulegen_ms_per_scan": kern["rulegen_ms"],
-        "streams": args.streams, "one_stream_ms_per_step": one_stream_ms,
-        "one_stream_value": n / (one_stream_ms * 1e-3),
-        "repeats": repeats,
-        "kernels": kern,
-        "roofline": wl.roofline(kern, args.seed),
+        "streams": args.streams,
+        "one_stream_value": n / (rep["one_stream_ms_per_step"] * 1e-3),
+        "host_value": n / (rep["host_ms_per_step"] * 1e-3),
     }
+    result.update({k: v for k, v in rep.items() if k != "ms_per_step"})
     if args.voxels > 0:
         # the size BASELINE's metric names: the same generator with its column occupancy raised
         d2, p2 = config2_with_voxels(args.voxels, seed=args.seed)
-        wl2, kern2, one2, ms2, rep2 = measure(d2)
+        wl2, kern2, t2 = measure(d2)
+        rep2 = report(wl2, kern2, t2)
         result["at_120k"] = {
             "workload": "config-2 generator with column occupancy %.3f: %d active voxels, %d pairs" % (p2, wl2.n, wl2.pairs),
-            "voxels": wl2.n, "pairs": wl2.pairs, "value": wl2.n / (ms2 * 1e-3), "unit": "voxels/s",
-            "ms_per_step": ms2, "one_stream_ms_per_step": one2, "rulegen_ms_per_scan": kern2["rulegen_ms"],
-            "kernels": kern2, "roofline": wl2.roofline(kern2, args.seed), "repeats": rep2}
+            "voxels": wl2.n, "pairs": wl2.pairs, "value": wl2.n / (rep2["ms_per_step"] * 1e-3), "unit": "voxels/s"}
+        result["at_120k"].update(rep2)
     if args.callers:
         result["callers"] = callers_ms(torch, d, args.seed, 50)
     if args.configs:

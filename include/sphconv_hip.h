@@ -115,10 +115,20 @@ int sph_num_tiles(const sph_geom *g, int T0, int T1);
  *                    grid), gathered side = input rows (z_idx/z_ptr over S).
  *   transposed == 1: stationary side = input rows, gathered side = output rows.
  * For a submanifold convolution pass the input arrays as the output arrays and
- * O == S.  `book.rows` must equal the stationary side's row count. */
+ * O == S.  `book.rows` must equal the stationary side's row count.
+ * row_cols (may be null): the column (flattened (b,s0,s1) index into the stationary side's pointer
+ * array) of every stationary row, as sph_row_columns, sph_init_tensor and sph_outcoords_fill write it.
+ * The reference gets a row's column for free from its launch geometry (one thread per column,
+ * rules.cu:256-259); here the tile workgroups otherwise search the pointer array for it.  Every
+ * entry is checked against the pointer array before it is believed: a wrong table costs time and
+ * cannot change the result. */
 int sph_rules_build(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
                     const int32_t *oz_idx, const int32_t *oz_ptr, int out_rows,
-                    const sph_geom *g, int transposed, const sph_book *book, void *stream);
+                    const sph_geom *g, int transposed, const sph_book *book,
+                    const int32_t *row_cols, void *stream);
+/* row_cols[r] = column of row r, from the inclusive pointer array z_ptr [ncol] (the expansion the
+ * reference's one-thread-per-column kernels never need, rules.cu:256-259). */
+int sph_row_columns(const int32_t *z_ptr, int ncol, int rows, int32_t *row_cols, void *stream);
 /* sph_rules_build with a weight pack (sph_weight_pack, same arguments) riding along as extra
  * workgroups of the same launch: for a layer whose rules are not cached yet, the forward pass
  * then is two launches (rules + pack, convolution) instead of three.  No reference counterpart
@@ -126,6 +136,7 @@ int sph_rules_build(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
 int sph_rules_build_pack(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
                          const int32_t *oz_idx, const int32_t *oz_ptr, int out_rows,
                          const sph_geom *g, int transposed, const sph_book *book,
+                         const int32_t *row_cols,
                          sph_dtype dt, const void *w, int KV, int kdim, int ndim, long stride_k,
                          long stride_kk, long stride_n, void *packed, void *stream);
 
@@ -142,7 +153,8 @@ int sph_rules_build_pack(const int32_t *z_idx, const int32_t *z_ptr, int in_rows
  *     Behind the state, when O[2] <= 512, each column's 64-bit masks of active bins (one per 64 bins) are
  *     kept for step 2; deeper grids keep none and step 2 walks the fibers again.
  *  2. once the caller knows the total: sph_outcoords_fill, given the same scratch and oz_ptr, writes
- *     oz_idx (ascending within a column).
+ *     oz_idx (ascending within a column) and, when row_cols is not null, every output row's column
+ *     (out_rows entries: the table sph_rules_build* takes for a layer that is stationary on these rows).
  * sph_outcoords_blocks(g) = ceil(columns / 256), the grid of the fill kernel. */
 int sph_outcoords_blocks(const sph_geom *g);
 int sph_outcoords_scratch_ints(const sph_geom *g);
@@ -152,7 +164,7 @@ int sph_outcoords_count(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
                         int32_t *total_dev, void *stream);
 int sph_outcoords_fill(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
                        const sph_geom *g, const int32_t *scratch, int32_t *oz_ptr,
-                       int32_t *oz_idx, int out_rows, void *stream);
+                       int32_t *oz_idx, int out_rows, int32_t *row_cols, void *stream);
 
 /* sph_outcoords_count for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
@@ -211,6 +223,20 @@ typedef struct sph_epilogue {
 int sph_conv_apply(sph_dtype dt, const void *feature, int feature_rows, int kdim,
                    const void *packed_w, int ndim, const sph_book *book,
                    const sph_epilogue *epi, void *out, void *stream);
+
+/* get_rules_subm / get_rules' pair half (rules.cu:326-390, 445-485) and rule_conv (rule_conv.cu:286-336) of ONE
+ * layer in ONE launch: every workgroup builds its tile's pairs in LDS as sph_rules_build does and convolves them
+ * at once as sph_conv_apply does; `out` [out_rows, ndim] is fully overwritten.  Arguments as for sph_rules_build
+ * (transposed == 0) and sph_conv_apply.  `book` must provide all group arrays: with write_book != 0 the book is
+ * filled as sph_rules_build fills it (for layers that share it through an indice_key, or for a backward pass);
+ * with write_book == 0 only tiles whose groups do not fit the workgroup's LDS (more than 64 groups) use their
+ * part of it, and its contents are unspecified afterwards.  Returns SPH_ERR_UNSUPPORTED (nothing launched) for
+ * shapes the fused kernel does not take -- rows that are not 16-byte multiples of up to 128 bytes, more than 64
+ * output channels, more than 32 kernel offsets: call sph_rules_build + sph_conv_apply then. */
+int sph_rules_conv(const int32_t *z_idx, const int32_t *z_ptr, int in_rows, const int32_t *oz_idx,
+                   const int32_t *oz_ptr, int out_rows, const sph_geom *g, const sph_book *book, int write_book,
+                   const int32_t *row_cols, sph_dtype dt, const void *feature, int kdim, const void *packed_w,
+                   int ndim, const sph_epilogue *epi, void *out, void *stream);
 
 /* Replaces rule_conv_d_weight (rule_conv.cu:469-518):
  *   d_weight[k, ci, co] = sum over pairs (k, in, out) feature[in, ci] * d_out[out, co]

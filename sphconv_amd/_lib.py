@@ -18,6 +18,7 @@ GROUP = 16
 STATIC_MAX_COLUMNS = 1 << 20     # SPH_STATIC_MAX_COLUMNS of the header
 
 F32, F16, BF16, I8 = 0, 1, 2, 3
+ERR_ARG, ERR_UNSUPPORTED, ERR_LAUNCH = -1, -2, -3      # sph_status
 _DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.int8: I8}
 
 
@@ -42,7 +43,7 @@ class Epilogue(C.Structure):
 
 
 _lib = None
-ABI_VERSION = 5       # sph_abi_version() of the library these signatures describe
+ABI_VERSION = 6       # sph_abi_version() of the library these signatures describe
 
 _I, _P, _L, _Z = C.c_int, C.c_void_p, C.c_long, C.c_size_t
 _SIGNATURES = {
@@ -52,21 +53,24 @@ _SIGNATURES = {
     "sph_book_cap": (_I, [_I]),
     "sph_tile_n_max": (_I, [C.POINTER(Geom), _I, _I, _I]),
     "sph_num_tiles": (_I, [C.POINTER(Geom), _I, _I]),
-    "sph_rules_build": (_I, [_P, _P, _I, _P, _P, _I, C.POINTER(Geom), _I, C.POINTER(Book), _P]),
-    "sph_rules_build_pack": (_I, [_P, _P, _I, _P, _P, _I, C.POINTER(Geom), _I, C.POINTER(Book), _I, _P, _I, _I, _I, _L, _L,
-                                  _L, _P, _P]),
+    "sph_rules_build": (_I, [_P, _P, _I, _P, _P, _I, C.POINTER(Geom), _I, C.POINTER(Book), _P, _P]),
+    "sph_rules_build_pack": (_I, [_P, _P, _I, _P, _P, _I, C.POINTER(Geom), _I, C.POINTER(Book), _P, _I, _P, _I, _I, _I, _L,
+                                  _L, _L, _P, _P]),
+    "sph_row_columns": (_I, [_P, _I, _I, _P, _P]),
     "sph_outcoords_blocks": (_I, [C.POINTER(Geom)]),
     "sph_outcoords_scratch_ints": (_I, [C.POINTER(Geom)]),
     "sph_outcoords_state_ints": (_I, [C.POINTER(Geom)]),
     "sph_outcoords_count": (_I, [_P, _P, _I, C.POINTER(Geom), _P, _P, _P, _P]),
     "sph_outcoords_count_static": (_I, [_P, _P, _I, C.POINTER(Geom), _P, _P, C.POINTER(C.c_void_p), _P]),
-    "sph_outcoords_fill": (_I, [_P, _P, _I, C.POINTER(Geom), _P, _P, _P, _I, _P]),
+    "sph_outcoords_fill": (_I, [_P, _P, _I, C.POINTER(Geom), _P, _P, _P, _I, _P, _P]),
     "sph_rules_to_padded_count": (_I, [C.POINTER(Book), _P, C.POINTER(Geom), _I, _I, _P, _P, _P]),
     "sph_rules_to_padded_fill": (_I, [_P, C.POINTER(Geom), _I, _I, _P, _I, _I, _I, _P, _P]),
     "sph_rules_from_padded": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _P, C.POINTER(Book), _P]),
     "sph_weight_packed_bytes": (_Z, [_I, _I, _I, _I]),
     "sph_weight_pack": (_I, [_I, _P, _I, _I, _I, _L, _L, _L, _P, _P]),
     "sph_conv_apply": (_I, [_I, _P, _I, _I, _P, _I, C.POINTER(Book), C.POINTER(Epilogue), _P, _P]),
+    "sph_rules_conv": (_I, [_P, _P, _I, _P, _P, _I, C.POINTER(Geom), C.POINTER(Book), _I, _P, _I, _P, _I, _P, _I,
+                            C.POINTER(Epilogue), _P, _P]),
     "sph_wgrad_partial_elems": (_Z, [_I, _I, _I, _I]),
     "sph_conv_wgrad": (_I, [_I, _P, _I, _I, _P, _I, C.POINTER(Book), _P, _P, _I, _P]),
     "sph_init_tensor_workspace": (_Z, [_I, _I, _I, _I, _I]),

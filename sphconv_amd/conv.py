@@ -53,6 +53,12 @@ class Convolution(SphModule):
             bound = 1 / math.sqrt(fan_in)
             nn.init.uniform_(self.bias, -bound, bound)
 
+    def invalidate_packed(self):
+        """Forgets the fragment-ordered copy of the weight that forward passes in eval mode keep under
+        ``torch.no_grad()``.  In-place updates that bump the weight's version counter (optimizer steps,
+        ``load_state_dict``, ``weight.mul_()``) are followed without this; updates through ``weight.data`` are not."""
+        ext.invalidate_packed(self.weight)
+
     @property
     def rule_size(self):
         """``rule_size [NTile,KV]`` of the last forward in the reference's format
@@ -99,29 +105,29 @@ class Conv3d(Convolution):
         return RuleBook.count_ahead(input.z_idx, input.z_ptr, input.B, in_shape, out_shape, self.kernel_size,
                                     self.stride, self.padding, self.dilation)
 
-    def _rules(self, input: SparseConvTensor, out_shape, weight=None, ahead=None):
+    def _rules(self, input: SparseConvTensor, out_shape, ahead=None, keep: bool = True):
         """Rule book of this layer on ``input``, shared through ``rule_cache`` when an
-        ``indice_key`` is set (conv.py:159-177).  Returns the cache entry and, when the
-        rules had to be generated, the weight packed by the same launch (else None)."""
+        ``indice_key`` is set (conv.py:159-177).  A book that is not cached yet is returned unbuilt (for a strided
+        layer with its output coordinates): ``rule_conv`` generates its pairs in the launch that convolves them
+        where that is faster, and otherwise, like every later use, builds it; ``keep``: that launch also writes
+        the book (later layers share it, or a backward pass follows)."""
         cached = input.find_rule(self.indice_key)
         if cached is not None:
-            return cached, None
+            return cached
         in_shape = [input.D, input.W, input.H]
-        if weight is not None and weight.dtype != input.feature.dtype:
-            weight = None
+        row_cols = getattr(input, "row_cols", None)
         if self.subm:
             book = RuleBook.build_subm(input.z_idx, input.z_ptr, input.B, in_shape, self.kernel_size,
-                                       self.padding, self.dilation, weight=weight)
+                                       self.padding, self.dilation, row_cols=row_cols, lazy=True)
         else:
             book = RuleBook.build(input.z_idx, input.z_ptr, input.B, in_shape, out_shape,
-                                  self.kernel_size, self.stride, self.padding, self.dilation, weight=weight, ahead=ahead)
-        packed = None
-        if weight is not None:
-            book, packed = book
+                                  self.kernel_size, self.stride, self.padding, self.dilation, ahead=ahead,
+                                  row_cols=row_cols, lazy=True)
+        book.keep = bool(keep)
         entry = (book.oz_idx, book.oz_ptr, book, None, get_tile_grid_shape(out_shape, self.tile_size))
         if self.indice_key is not None:
             input.rule_cache[self.indice_key] = entry
-        return entry, packed
+        return entry
 
     def forward(self, input: SparseConvTensor, epilogue=None, ahead=None) -> SparseConvTensor:
         """``epilogue`` = (scale [oC] fp32 or None, shift [oC] fp32 or None, relu): applied to the
@@ -134,20 +140,29 @@ class Conv3d(Convolution):
         out_shape = in_shape if self.subm else out_spatial(in_shape, self.kernel_size, self.stride,
                                                             self.padding, self.dilation)
         weight = self.weight.view(-1, self.in_channels, self.out_channels)
-        (oz_idx, oz_ptr, book, rule_size, tile_grid_shape), packed = self._rules(input, out_shape, weight, ahead)
+        training = torch.is_grad_enabled() and (weight.requires_grad or input.feature.requires_grad)
+        oz_idx, oz_ptr, book, rule_size, tile_grid_shape = self._rules(
+            input, out_shape, ahead, keep=training or self.indice_key is not None)
         self.rule_book = book if isinstance(book, RuleBook) else None
         if epilogue is not None:
-            if torch.is_grad_enabled() and (weight.requires_grad or input.feature.requires_grad):
+            if training:
                 raise RuntimeError("a fused epilogue has no backward: call under torch.no_grad()")
             scale, shift, relu = epilogue
             w = weight if weight.dtype == input.feature.dtype else weight.to(input.feature.dtype)
             out_feature = ext.rule_conv(input.feature, w, book, rule_size, oz_idx.shape[0], scale, shift,
-                                        bool(relu), packed if w is weight else None)
+                                        bool(relu), cache_packed=not self.training and w is weight)
+        elif not training:
+            w = weight if weight.dtype == input.feature.dtype else weight.to(input.feature.dtype)
+            out_feature = ext.rule_conv(input.feature, w.detach(), book, rule_size, oz_idx.shape[0],
+                                        cache_packed=not self.training and w is weight)
         else:
             out_feature = ConvFunction.apply(input.feature, weight, book, rule_size, tile_grid_shape,
-                                             oz_idx.shape[0], packed)
+                                             oz_idx.shape[0])
         out = SparseConvTensor(out_feature, out_shape, input.B, z_ptr=oz_ptr, z_idx=oz_idx)
         out.rule_cache = input.rule_cache
+        # the rows' columns, where known: the input's own for a submanifold layer, a by-product of the
+        # output-coordinate kernels for a strided one
+        out.row_cols = book.out_row_cols if isinstance(book, RuleBook) else None
         return out
 
 

@@ -21,70 +21,11 @@
 // that are not whole 16-byte chunks.
 #include "common.h"
 #include "pack.h"
+#include "conv_wave.h"
+
+#include <cstdlib>
 
 namespace {
-
-constexpr int R = SPH_TILE_ROWS;
-constexpr int kWave = 64;
-
-typedef int int4v __attribute__((ext_vector_type(4)));
-typedef float float4v __attribute__((ext_vector_type(4)));
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
-
-template <sph_dtype DT> struct Traits;
-template <> struct Traits<SPH_F32> {
-    typedef float elem;
-    typedef float4v acc4;
-    static constexpr int KW = 4; // elements per 16-byte fragment
-};
-template <> struct Traits<SPH_F16> {
-    typedef _Float16 elem;
-    typedef float4v acc4;
-    static constexpr int KW = 8;
-};
-template <> struct Traits<SPH_BF16> {
-    typedef __bf16 elem;
-    typedef float4v acc4;
-    static constexpr int KW = 8;
-};
-template <> struct Traits<SPH_I8> {
-    typedef int8_t elem;
-    typedef int4v acc4;
-    static constexpr int KW = 16;
-};
-
-// One "super step" consumes 64 bytes of every gathered row: lane l supplies the
-// 16 bytes at offset 16*(l/16) of row l%16 (A) / of column l%16 (B).  Any
-// assignment of K indices to lanes is valid as long as A and B agree.
-template <sph_dtype DT>
-__device__ __forceinline__ typename Traits<DT>::acc4 mfma_step(int4v a, int4v b, typename Traits<DT>::acc4 d);
-
-template <>
-__device__ __forceinline__ float4v mfma_step<SPH_F32>(int4v a, int4v b, float4v d)
-{
-    const float4v af = __builtin_bit_cast(float4v, a), bf = __builtin_bit_cast(float4v, b);
-    d = __builtin_amdgcn_mfma_f32_16x16x4f32(af.x, bf.x, d, 0, 0, 0);
-    d = __builtin_amdgcn_mfma_f32_16x16x4f32(af.y, bf.y, d, 0, 0, 0);
-    d = __builtin_amdgcn_mfma_f32_16x16x4f32(af.z, bf.z, d, 0, 0, 0);
-    d = __builtin_amdgcn_mfma_f32_16x16x4f32(af.w, bf.w, d, 0, 0, 0);
-    return d;
-}
-template <>
-__device__ __forceinline__ float4v mfma_step<SPH_F16>(int4v a, int4v b, float4v d)
-{
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), d, 0, 0, 0);
-}
-template <>
-__device__ __forceinline__ float4v mfma_step<SPH_BF16>(int4v a, int4v b, float4v d)
-{
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, a), __builtin_bit_cast(bf8, b), d, 0, 0, 0);
-}
-template <>
-__device__ __forceinline__ int4v mfma_step<SPH_I8>(int4v a, int4v b, int4v d)
-{
-    return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, d, 0, 0, 0);
-}
 
 // ---------------------------------------------------------------------------
 // Weight packing (layout and element copy: pack.h)
@@ -92,91 +33,6 @@ __device__ __forceinline__ int4v mfma_step<SPH_I8>(int4v a, int4v b, int4v d)
 __global__ void pack_weight_kernel(SphPackJob p)
 {
     sph_pack_element(p, (long)blockIdx.x * blockDim.x + threadIdx.x);
-}
-
-struct ConvArgs {
-    const char *feat;
-    int feat_rows, kdim, row_bytes;
-    const char *wp;
-    int nsteps, ndim;
-    sph_book book;
-    int cap;
-    const float *scale, *shift;
-    int relu;
-    char *out;
-    int aligned_in, aligned_out;
-};
-
-// can sph_conv_apply walk this call by stationary row?
-inline bool rows_path_ok(const ConvArgs &a)
-{
-    return a.aligned_in && a.aligned_out && a.feat_rows > 0 && a.book.tile_nbr && (a.nsteps == 1 || a.nsteps == 2) &&
-           (size_t)a.book.KV * R * sizeof(int32_t) <= 48 * 1024 && (uintptr_t)a.book.tile_nbr % 16 == 0;
-}
-
-template <sph_dtype DT>
-__device__ __forceinline__ int4v load_a_frag(const ConvArgs &a, int in_row, int st, int lane)
-{
-    typedef typename Traits<DT>::elem elem;
-    constexpr int KW = Traits<DT>::KW;
-    int4v f = {0, 0, 0, 0};
-    if ((unsigned)in_row >= (unsigned)a.feat_rows) return f;
-    const int byte_off = st * 64 + (lane >> 4) * 16;
-    const char *row = a.feat + (long)in_row * a.row_bytes;
-    if (a.aligned_in) {
-        if (byte_off < a.row_bytes) f = *(const int4v *)(row + byte_off);
-    } else {
-        union { int4v v; elem e[KW]; } u;
-        u.v = f;
-        const int c0 = byte_off / (int)sizeof(elem);
-#pragma unroll
-        for (int j = 0; j < KW; j++)
-            if (c0 + j < a.kdim) u.e[j] = ((const elem *)row)[c0 + j];
-        f = u.v;
-    }
-    return f;
-}
-
-template <sph_dtype DT>
-__device__ __forceinline__ float epilogue_value(const ConvArgs &a, uint32_t raw, int c)
-{
-    float v;
-    if (DT == SPH_I8)
-        v = (float)(int32_t)raw;
-    else
-        v = __builtin_bit_cast(float, raw);
-    if (a.scale) v = v * a.scale[c];
-    if (DT != SPH_I8) {
-        if (a.shift) v = v + a.shift[c];
-        if (a.relu) v = v > 0.f ? v : 0.f;
-    }
-    return v;
-}
-
-template <sph_dtype DT>
-__device__ __forceinline__ typename Traits<DT>::elem to_elem(float v)
-{
-    typedef typename Traits<DT>::elem elem;
-    if (DT == SPH_I8) {
-        float r = __builtin_rintf(v);
-        r = r < -128.f ? -128.f : (r > 127.f ? 127.f : r);
-        return (elem)(int)r;
-    }
-    return (elem)v;
-}
-
-// Adds the four accumulators a lane holds after a transposed MFMA (four consecutive
-// output columns of ONE owner row) into the LDS tile with a single 16-byte
-// read-modify-write.  The address range belongs to this wave only, so additions
-// happen in program order and the sum is reproducible.  (LDS float atomics
-// serialise per lane and measured 2x slower.)
-template <sph_dtype DT>
-__device__ __forceinline__ void acc_add4(uint32_t *p, typename Traits<DT>::acc4 d)
-{
-    typedef typename Traits<DT>::acc4 acc4;
-    acc4 v = *(acc4 *)p;
-    v += d;
-    *(acc4 *)p = v;
 }
 
 constexpr int kMetaGroups = 32; // groups whose indices are staged in LDS at a time
@@ -266,31 +122,11 @@ __global__ __launch_bounds__(NW * kWave) void conv_apply_kernel(ConvArgs a)
 }
 
 // ---------------------------------------------------------------------------
-// One wave per tile and per block of 64 output columns.
-//
-// At LiDAR sizes (a few hundred tiles) every workgroup of the grid is resident at
-// once, so the kernel lasts as long as ONE tile's dependent chain; barriers and
-// fragment exchange between waves only lengthen that chain.  Here a wave owns a
-// tile (x 64 columns) outright: it gathers each group's rows once (16 B per lane,
-// already MFMA operand order), loads the offset's weight fragments, and accumulates
-// into its own LDS tile: the accumulator rows of the group's owners are read as the
-// C operand of the MFMAs and written back.  No barrier, no atomics, summation order
-// = book order.  Indices run two blocks ahead; gathers and weight fragments are
-// requested three to four groups before their use, their address arithmetic is
-// interleaved with the MFMAs.  Measured bounds of the loop at 64->64 fp16: the
-// vector-memory return path (8 KiB of weight fragments + 2 KiB of rows per group),
-// then the LDS read-MFMA-write chain, then the MFMAs themselves.
-// ---------------------------------------------------------------------------
-constexpr int kBlk = 4; // groups per pipeline block (4 x 16 index entries = one 64-lane load)
 
 template <sph_dtype DT, int NS, int CT, bool MASKED>
 __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
 {
-    typedef typename Traits<DT>::elem elem;
-    typedef typename Traits<DT>::acc4 acc4;
-    extern __shared__ __attribute__((aligned(16))) uint32_t s_acc[]; // [R][LDW]
-    const int LDW = nwtot * 16 + 4;
-
+    extern __shared__ __attribute__((aligned(16))) uint32_t s_acc[]; // [R + 1][LDW]
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;              // block of CT*16 columns
@@ -299,233 +135,10 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
     if (r0 >= a.book.rows) return;
     const int nrows = min(R, a.book.rows - r0);
     const int col0 = wave * CT * 16;           // first column of this wave
-
     const int ngrp = a.book.tile_ngrp[tile];
-    const long gb0 = (long)tile * a.cap;
-    // Every load of the loop goes through a buffer descriptor: the address is a scalar base plus a 32-bit lane
-    // offset (plus a scalar offset for the weight's kernel offset), so no load costs 64-bit vector arithmetic,
-    // and a read beyond the array returns zeros instead of faulting.  (The launcher sends arrays of 4 GiB or more
-    // to the general kernel.)
-    constexpr int kRsrcFlags = 0x00020000; // raw buffer, 32-bit data format
-    const __amdgpu_buffer_rsrc_t r_gat = __builtin_amdgcn_make_buffer_rsrc((void *)(a.book.grp_gather + gb0 * SPH_GROUP), 0,
-                                                                           a.cap * SPH_GROUP * 4, kRsrcFlags);
-    const __amdgpu_buffer_rsrc_t r_own = __builtin_amdgcn_make_buffer_rsrc((void *)(a.book.grp_owner + gb0 * SPH_GROUP), 0,
-                                                                           a.cap * SPH_GROUP * 4, kRsrcFlags);
-    const __amdgpu_buffer_rsrc_t r_gk = __builtin_amdgcn_make_buffer_rsrc((void *)(a.book.grp_k + gb0), 0, a.cap * 4, kRsrcFlags);
-    const __amdgpu_buffer_rsrc_t r_feat = __builtin_amdgcn_make_buffer_rsrc((void *)a.feat, 0, a.feat_rows * a.row_bytes, kRsrcFlags);
-    // weight fragment of (offset k, step st, column tile c): k*NS*nwtot + st*nwtot + c  (1 KiB each)
-    const int wstep = nwtot * (kWave * 16);
-    const __amdgpu_buffer_rsrc_t r_w = __builtin_amdgcn_make_buffer_rsrc((void *)a.wp, 0, a.book.KV * NS * wstep, kRsrcFlags);
-    int woff[NS]; // lane offset of the wave's first column tile at step st
-#pragma unroll
-    for (int st = 0; st < NS; st++) woff[st] = st * wstep + (wave * CT) * (kWave * 16) + lane * 16;
-    const int lane_chunk = (lane >> 4) * 16;
-
-    // Every load below is unconditional and straight-line (indices are clamped to
-    // memory that is always allocated, results of invalid slots are discarded by
-    // selects): the compiler can then count outstanding loads exactly and only waits
-    // for the ones an instruction needs.
-    // Index loads return raw values; they are validated (finish_meta) only when the block
-    // is about to be used, one or two blocks later -- touching a loaded value earlier
-    // would make the wave wait for it, and with it for every load issued before.
-    auto load_meta = [&](int g0, int &gi, int &ow, int &kk) {
-        // one load each: lane l holds entry l%16 of group g0 + l/16; lanes 0..3 hold the offsets
-        const int gs = min(g0, a.cap - kBlk); // stay inside this tile's capacity
-        gi = __builtin_amdgcn_raw_buffer_load_b32(r_gat, lane * 4, gs * (SPH_GROUP * 4), 0);
-        ow = __builtin_amdgcn_raw_buffer_load_b32(r_own, lane * 4, gs * (SPH_GROUP * 4), 0);
-        kk = __builtin_amdgcn_raw_buffer_load_b32(r_gk, (lane & (kBlk - 1)) * 4, gs * 4, 0);
-    };
-    auto finish_meta = [&](int g0, int &gi, int &ow, int &kk) {
-        const bool inside = g0 <= a.cap - kBlk;
-        const int g = g0 + (lane >> 4);
-        const int vow = ow - r0;
-        const bool ok = inside && g < ngrp && (unsigned)vow < (unsigned)nrows && (unsigned)gi < (unsigned)a.feat_rows;
-        gi = ok ? gi : -1;
-        ow = ok ? vow : -1;
-        kk = (inside && g0 + (lane & (kBlk - 1)) < ngrp && (unsigned)kk < (unsigned)a.book.KV) ? kk : 0;
-    };
-    // Gathers only load (from an address clamped into the feature array); slots that hold
-    // no pair and the tail of rows shorter than the step are zeroed when the fragment is
-    // used, not here -- a select on the loaded value would stall the wave on the load.
-    auto load_a = [&](int gi_blk, int u, int4v (&fa)[NS]) {
-        const int in_row = __shfl(gi_blk, u * SPH_GROUP + (lane & 15), kWave);
-        const int row = max(in_row, 0) * a.row_bytes + lane_chunk;   // a row shorter than the step: the tail is the next row's, masked later
-#pragma unroll
-        for (int st = 0; st < NS; st++)
-            fa[st] = __builtin_bit_cast(int4v, __builtin_amdgcn_raw_buffer_load_b128(r_feat, row + st * 64, 0, 0));
-    };
-    auto load_w = [&](int k, int4v (&fw)[NS][CT]) {
-        const int wk = k * (NS * wstep); // scalar
-#pragma unroll
-        for (int st = 0; st < NS; st++)
-#pragma unroll
-            for (int c = 0; c < CT; c++)
-                fw[st][c] = __builtin_bit_cast(int4v, __builtin_amdgcn_raw_buffer_load_b128(r_w, woff[st] + c * (kWave * 16), wk, 0));
-    };
-    // Accumulator address of a pair: its owner's row, or the scratch row behind the tile for
-    // a padding slot (which multiplies whatever row 0 holds): no branch, no select on data.
-    auto acc_ptr = [&](int ow_blk, int u) -> uint32_t * {
-        const int rl = __shfl(ow_blk, u * SPH_GROUP + (lane & 15), kWave);
-        return &s_acc[(rl >= 0 ? rl : R) * LDW + col0 + (lane >> 4) * 4];
-    };
-    // One group: the accumulator rows are requested first and are the C operand of the
-    // MFMAs (the matrix unit does the addition); the next weight fragments are requested
-    // while they arrive; once the MFMAs have consumed this group's gathered rows, the same
-    // registers take the gather of the same slot of the next block.
-    auto group_step = [&](const int4v (&fw)[NS][CT], int4v (&fa)[NS], uint32_t *p, int k_next, int4v (&fw_next)[NS][CT],
-                          int gi_next, int u) {
-        acc4 d[CT];
-#pragma unroll
-        for (int c = 0; c < CT; c++) d[c] = *(const acc4 *)(p + c * 16);
-        __builtin_amdgcn_sched_barrier(0);
-        load_w(k_next, fw_next);
-        if constexpr (MASKED) { // rows shorter than the steps, e.g. 4 fp32 channels = 16 of 64 bytes: zero the tail
-#pragma unroll
-            for (int st = 0; st < NS; st++) {
-                const bool live = st * 64 + (lane >> 4) * 16 < a.row_bytes;
-                const int4v x = live ? fa[st] : int4v{0, 0, 0, 0};
-#pragma unroll
-                for (int c = 0; c < CT; c++) d[c] = mfma_step<DT>(fw[st][c], x, d[c]);
-            }
-        } else {
-#pragma unroll
-            for (int st = 0; st < NS; st++)
-#pragma unroll
-                for (int c = 0; c < CT; c++) d[c] = mfma_step<DT>(fw[st][c], fa[st], d[c]);
-        }
-        load_a(gi_next, u, fa);
-#pragma unroll
-        for (int c = 0; c < CT; c++) *(acc4 *)(p + c * 16) = d[c];
-#pragma unroll
-        for (int i = 0; i < NS * CT; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
-            __builtin_amdgcn_sched_group_barrier(0x006, 3, 0); // VALU / SALU
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // one VMEM read
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    // Pipeline: indices run two blocks ahead; the gathers of slot u and the weight
-    // fragments of a group are requested three to four groups before their use.
-    int gi_n, ow_n, k_n;       // indices of the next block
-    int gi_nn, ow_nn, k_nn;    // indices of the block after it
-    int4v a_0[NS], a_1[NS], a_2[NS], a_3[NS];                 // gathered rows of slot u
-    int4v w_0[NS][CT], w_1[NS][CT], w_2[NS][CT], w_3[NS][CT]; // fragments for group u of a block live in w_u
-    int ow_c, k_c;
-
-    load_meta(0, gi_n, ow_n, k_n);
-    load_meta(kBlk, gi_nn, ow_nn, k_nn);
-    // clear the accumulator tile (and the scratch row) while the first indices are on their way
-    for (int i = lane; i < (R + 1) * CT * 4; i += kWave)
-        *(int4v *)&s_acc[(i / (CT * 4)) * LDW + col0 + (i % (CT * 4)) * 4] = int4v{0, 0, 0, 0};
-    finish_meta(0, gi_n, ow_n, k_n);
-    // The first loads are issued in the order the loop issues them (rows of slot u, then the fragments of group u),
-    // pinned against the scheduler: the compiler places one wait count per use for every path into the loop, and a
-    // start that had requested the first group's fragments last would make every block of the loop wait for all but
-    // its last ten loads (the loop's own order lets about thirty stay in flight).
-    load_a(gi_n, 0, a_0);
-    __builtin_amdgcn_sched_barrier(0);
-    load_w(__builtin_amdgcn_readlane(k_n, 0), w_0);
-    __builtin_amdgcn_sched_barrier(0);
-    load_a(gi_n, 1, a_1);
-    __builtin_amdgcn_sched_barrier(0);
-    load_w(__builtin_amdgcn_readlane(k_n, 1), w_1);
-    __builtin_amdgcn_sched_barrier(0);
-    load_a(gi_n, 2, a_2);
-    __builtin_amdgcn_sched_barrier(0);
-    load_w(__builtin_amdgcn_readlane(k_n, 2), w_2);
-    __builtin_amdgcn_sched_barrier(0);
-    load_a(gi_n, 3, a_3);
-    __builtin_amdgcn_sched_barrier(0);
-
-    for (int g0 = 0; g0 < ngrp; g0 += kBlk) {
-        ow_c = ow_n; k_c = k_n;
-        gi_n = gi_nn; ow_n = ow_nn; k_n = k_nn;
-        finish_meta(g0 + kBlk, gi_n, ow_n, k_n);   // loaded one block ago
-        load_meta(g0 + 2 * kBlk, gi_nn, ow_nn, k_nn);
-        uint32_t *p_0 = acc_ptr(ow_c, 0), *p_1 = acc_ptr(ow_c, 1), *p_2 = acc_ptr(ow_c, 2), *p_3 = acc_ptr(ow_c, 3);
-        __builtin_amdgcn_sched_barrier(0);
-        group_step(w_0, a_0, p_0, __builtin_amdgcn_readlane(k_c, 3), w_3, gi_n, 0);
-        group_step(w_1, a_1, p_1, __builtin_amdgcn_readlane(k_n, 0), w_0, gi_n, 1);
-        group_step(w_2, a_2, p_2, __builtin_amdgcn_readlane(k_n, 1), w_1, gi_n, 2);
-        group_step(w_3, a_3, p_3, __builtin_amdgcn_readlane(k_n, 2), w_2, gi_n, 3);
-    }
-
-    // epilogue: this wave's columns of rows [r0, r0+nrows)
-    constexpr int VE = 16 / (int)sizeof(elem);
-    const int ncols = min(CT * 16, a.ndim - col0);
-    if (ncols <= 0) return;
-    elem *out = (elem *)a.out + (long)r0 * a.ndim + col0;
-    const bool plain = DT != SPH_I8 && !a.scale && !a.shift && !a.relu;
-    if (a.aligned_out && ncols % VE == 0) {
-        // lane = (row within a pass, 16-byte chunk of the row): VE accumulators -> one 16-byte store
-        const int cpr = ncols / VE;                 // chunks per row (power of two here)
-        const int ch = lane % cpr, rstep = kWave / cpr;
-        if (plain) {
-            // four rows per pass: their LDS reads are all issued before the first conversion
-            constexpr int UR = 4;
-            for (int row0 = lane / cpr; row0 < nrows; row0 += UR * rstep) {
-                float4v f[UR][VE / 4];
-#pragma unroll
-                for (int q = 0; q < UR; q++) {
-                    const int row = min(row0 + q * rstep, nrows - 1);
-#pragma unroll
-                    for (int j = 0; j < VE / 4; j++)
-                        f[q][j] = *(const float4v *)&s_acc[row * LDW + col0 + ch * VE + j * 4];
-                }
-#pragma unroll
-                for (int q = 0; q < UR; q++) {
-                    const int row = row0 + q * rstep;
-                    union { int4v v; elem e[VE]; } u;
-#pragma unroll
-                    for (int j = 0; j < VE / 4; j++) {
-                        u.e[4 * j] = (elem)f[q][j].x; u.e[4 * j + 1] = (elem)f[q][j].y;
-                        u.e[4 * j + 2] = (elem)f[q][j].z; u.e[4 * j + 3] = (elem)f[q][j].w;
-                    }
-                    if (row < nrows) *(int4v *)(out + (long)row * a.ndim + ch * VE) = u.v;
-                }
-            }
-        } else {
-            // scale / shift of this lane's VE columns stay in registers for all rows
-            float sc[VE], sh[VE];
-#pragma unroll
-            for (int j = 0; j < VE; j++) {
-                sc[j] = a.scale ? a.scale[col0 + ch * VE + j] : 1.f;
-                sh[j] = (DT != SPH_I8 && a.shift) ? a.shift[col0 + ch * VE + j] : 0.f;
-            }
-            const bool relu = DT != SPH_I8 && a.relu;
-            constexpr int UR = VE > 8 ? 2 : 4;
-            for (int row0 = lane / cpr; row0 < nrows; row0 += UR * rstep) {
-                int4v f[UR][VE / 4];
-#pragma unroll
-                for (int q = 0; q < UR; q++) {
-                    const int row = min(row0 + q * rstep, nrows - 1);
-#pragma unroll
-                    for (int j = 0; j < VE / 4; j++)
-                        f[q][j] = *(const int4v *)&s_acc[row * LDW + col0 + ch * VE + j * 4];
-                }
-#pragma unroll
-                for (int q = 0; q < UR; q++) {
-                    const int row = row0 + q * rstep;
-                    union { int4v v; elem e[VE]; } u;
-#pragma unroll
-                    for (int j = 0; j < VE; j++) {
-                        const int raw = j % 4 == 0 ? f[q][j / 4].x : (j % 4 == 1 ? f[q][j / 4].y : (j % 4 == 2 ? f[q][j / 4].z : f[q][j / 4].w));
-                        float v = DT == SPH_I8 ? (float)raw : __builtin_bit_cast(float, raw);
-                        v = v * sc[j] + sh[j];
-                        if (relu) v = v > 0.f ? v : 0.f;
-                        u.e[j] = to_elem<DT>(v);
-                    }
-                    if (row < nrows) *(int4v *)(out + (long)row * a.ndim + ch * VE) = u.v;
-                }
-            }
-        }
-    } else {
-        for (int i = lane; i < nrows * ncols; i += kWave) {
-            int row = i / ncols, c = i - row * ncols;
-            out[(long)row * a.ndim + c] = to_elem<DT>(epilogue_value<DT>(a, s_acc[row * LDW + col0 + c], col0 + c));
-        }
-    }
+    const BookMeta meta(a.book, a.cap, tile, ngrp, r0, nrows, a.feat_rows);
+    conv_wave_groups<DT, NS, CT, MASKED>(a, nwtot, meta, ngrp, s_acc, col0, lane, true);
+    conv_wave_store<DT, CT>(a, nwtot, s_acc, col0, r0, nrows, lane, kWave);
 }
 
 // ---------------------------------------------------------------------------
@@ -1529,9 +1142,9 @@ template <sph_dtype DT, int NS, int CT, bool MASKED>
 int launch_conv_wave(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
 {
     size_t lds = (size_t)(R + 1) * (nwtot * 16 + 4) * sizeof(uint32_t); // + scratch row
+    const int waves = (nwtot + CT - 1) / CT;
     int rc = set_lds(conv_wave_kernel<DT, NS, CT, MASKED>, lds);
     if (rc) return rc;
-    const int waves = (nwtot + CT - 1) / CT;
     hipLaunchKernelGGL((conv_wave_kernel<DT, NS, CT, MASKED>), dim3(sph_xcd_grid(ntiles)), dim3(waves * kWave), lds, st, a, nwtot);
     return sph_check_launch("sph_conv_apply");
 }
@@ -1609,8 +1222,9 @@ int launch_conv(const ConvArgs &a, int ntiles, hipStream_t st)
         if (a.nsteps == 1) return launch_conv_rows_ct<DT, 1>(a, NW, ntiles, st);
         return launch_conv_rows_ct<DT, 2>(a, NW, ntiles, st);
     }
-    // the one-wave-per-tile kernel addresses the feature array through a buffer descriptor with 32-bit offsets
-    const bool small = (double)a.feat_rows * a.row_bytes < 2147483648.0;
+    // the one-wave-per-tile kernel addresses the feature array through a buffer descriptor with 31-bit offsets
+    // made by a 24-bit multiply
+    const bool small = (double)a.feat_rows * a.row_bytes < 2147483648.0 && a.feat_rows < (1 << 24);
     if (a.aligned_in && a.feat_rows > 0 && small) {
         switch (a.nsteps) {
         case 1: return launch_conv_wave_ct<DT, 1>(a, NW, ntiles, st);

@@ -2,8 +2,8 @@
 // convolution and the rule book of (kernel offset, gathered row, owner row)
 // triples, replacing the reference's dense [B,S0,S1,S2] position grid and
 // atomic counters (src/sphconv/rules.cu) by fiber joins, wave ballots and
-// prefix popcounts; the per-column output counts are scanned inside the kernel
-// that counts them (single pass, decoupled look-back between workgroups).
+// prefix popcounts; the per-column output counts are scanned by a second kernel
+// (scan.h: one pass over the counts, decoupled look-back between workgroups).
 // All kernels are integer and HBM/latency bound.
 #include "common.h"
 #include "pack.h"
@@ -12,305 +12,16 @@
 #include <cstring>
 #include <mutex>
 
+#include "rules_tile.h"
+
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kWave = 64;
-constexpr int kWaves = kThreads / kWave;
-constexpr int R = SPH_TILE_ROWS;
-
-struct Grid3 {
-    int n0, n1, n2;
-};
-
-// Division of a 32-bit unsigned number by a divisor fixed per launch: a multiplication and two shifts with
-// constants made on the host (Granlund and Montgomery's round-up method, exact for every 32-bit numerator),
-// where the compiler's division by a run-time value is some thirty instructions in a row.
-struct FastDiv {
-    uint32_t mul, sh1, sh2;
-};
-inline FastDiv fast_div(uint32_t d)
-{
-    uint32_t l = 0;
-    while ((1ull << l) < d) l++;
-    const uint32_t m = (uint32_t)((((1ull << l) - d) << 32) / d + 1);
-    return FastDiv{m, l < 1 ? l : 1, l < 1 ? 0 : l - 1};
-}
-__device__ __forceinline__ uint32_t div_by(uint32_t n, const FastDiv &f)
-{
-    const uint32_t t = __umulhi(f.mul, n);
-    return (t + ((n - t) >> f.sh1)) >> f.sh2;
-}
-
-struct ConvParams {
-    int K0, K1, K2;
-    int s0, s1, s2;
-    int p0, p1, p2;
-};
-
-// Barrier for data exchanged through LDS only.  __syncthreads() also waits for every global load and store of
-// the thread that is still in flight (a full memory round trip each time one is pending); the rule kernels
-// share nothing through global memory inside a workgroup, so their barriers order LDS accesses alone.
-__device__ __forceinline__ void lds_barrier()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
-__device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
-
-// Row range [start, end) of column c, clamped to [0, rows] so that inconsistent
-// caller data can never index outside the row arrays.
-__device__ __forceinline__ void fiber_range(const int32_t *ptr, int c, int rows, int &start, int &end)
-{
-    end = clampi(ptr[c], 0, rows);
-    start = c ? clampi(ptr[c - 1], 0, rows) : 0;
-    if (start > end) start = end;
-}
-
-// Narrows down the first column c in [0, n) with a[c] > target (n if none): returns
-// lo <= c with c - lo < max_span.  All kThreads threads of the block work together:
-// every round probes kThreads evenly spaced positions of the remaining window, so a
-// round cuts the window by a factor of kThreads.  (Probes are scattered, one cache
-// line each, and cost far more in the vector memory path than the coalesced column
-// walk that follows; hence few probes and an early stop.)  max_span = 1 gives the
-// exact column.  s_first: 2 * kWaves LDS ints (the rounds alternate between the halves,
-// so a round needs one barrier).  meanwhile() runs once, while the first round's probes are in flight,
-// and in front of a barrier: the place for LDS initialisation.  Must be called by the whole block.
-template <class F>
-__device__ int block_upper_bound(const int32_t *a, int n, int target, int max_span, int *s_first, F &&meanwhile)
-{
-    int lo = 0, hi = n;
-    const int tid = threadIdx.x;
-    bool first = true;
-    for (int round = 0; hi - lo >= max_span; round ^= 1) {
-        int span = hi - lo;
-        int step = (span + kThreads - 1) / kThreads;
-        long pos = (long)lo + (long)tid * step;
-        int val = (pos < hi) ? a[pos] : 0x7fffffff; // positions >= hi are known to exceed
-        if (first) meanwhile();
-        first = false;
-        // first probe above the target: per wave by a ballot, over the waves through LDS
-        const unsigned long long above = __ballot(val > target);
-        int *mine = s_first + round * kWaves;
-        if ((tid & (kWave - 1)) == 0) mine[tid / kWave] = above ? (tid & ~(kWave - 1)) + __ffsll((long long)above) - 1 : kThreads;
-        lds_barrier();
-        int f = kThreads;
-#pragma unroll
-        for (int w = 0; w < kWaves; w++) f = min(f, mine[w]);
-        if (f == kThreads) {
-            lo = lo + (kThreads - 1) * step + 1;
-        } else {
-            long nh = (long)lo + (long)f * step;
-            int new_hi = nh < hi ? (int)nh : hi;
-            int new_lo = (f == 0) ? lo : lo + (f - 1) * step + 1;
-            hi = new_hi;
-            lo = new_lo;
-        }
-    }
-    if (first) { // no round at all
-        meanwhile();
-        lds_barrier();
-    }
-    return lo;
-}
-
-// ---------------------------------------------------------------------------
-// Shared tail of the book builders: the block holds, in LDS, a table
-// nbr[row_local * KV + k] = gathered row or -1 for the R rows of tile `tile`
-// (first row r0; rows behind the tile's last one hold -1).  Emits the tile's
-// groups: per k, rows in ascending order, 16 per group, last group padded with -1.
-//   pass 1: a wave takes an offset k: two ballots over the column k of the table
-//           give every row with a pair its rank in the k-list, and the row writes
-//           its number into the list's place in LDS (sel[k][rank]);
-//   scan  : first group of every k, and one descriptor word per group;
-//   pass 2: one thread per output SLOT reads its group's descriptor, the row at its
-//           rank and the row's table entry, and stores -- consecutive threads store
-//           consecutive slots, so the book is written coalesced.
-// A tile's time is the length of its waves' dependent chains (the same with one
-// workgroup per CU as with three): every step above is a handful of instructions per
-// item, batched so that the LDS round trips of several items overlap.
-// ---------------------------------------------------------------------------
-// Lives in dynamic LDS behind the neighbour table, sized by the kernel volume (a 3x3x3 kernel needs 4.5 KB
-// where the largest volume needs 21 KB).
-struct EmitScratch {
-    int *cnt;           // [KV] pairs of offset k
-    int *goff;          // [KV + 1] first group of offset k
-    int *ginfo;         // [KV * (R / SPH_GROUP)] per group: k | rank of its first slot << 8 | cnt[k] << 16
-    unsigned char *sel; // [KV][R] rows of offset k's list
-};
-__host__ __device__ inline size_t emit_scratch_bytes(int KV)
-{
-    const size_t b = (size_t)KV * sizeof(int) + (size_t)(KV + 1) * sizeof(int) +
-                     (size_t)KV * (R / SPH_GROUP) * sizeof(int) + (size_t)KV * R;
-    return (b + 7) & ~(size_t)7;
-}
-// `base` must be 4-byte aligned.
-__device__ __forceinline__ EmitScratch emit_scratch_at(void *base, int KV)
-{
-    EmitScratch sc;
-    sc.cnt = (int *)base;
-    sc.goff = sc.cnt + KV;
-    sc.ginfo = sc.goff + KV + 1;
-    sc.sel = (unsigned char *)(sc.ginfo + KV * (R / SPH_GROUP));
-    return sc;
-}
-
-// Inclusive sum over the wave's 64 lanes through the data-parallel-primitive lane shifts of the vector ALU
-// (four shifts inside a row of 16 lanes, then lane 15 and lane 31 broadcast into the rows behind them):
-// no LDS round trip per step as a shuffle has.
-__device__ __forceinline__ int wave_inclusive_sum(int x)
-{
-    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, false); // row_shr:1
-    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, false); // row_shr:2
-    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, false); // row_shr:4
-    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, false); // row_shr:8
-    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, false); // row_bcast:15 into rows 1 and 3
-    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, false); // row_bcast:31 into rows 2 and 3
-    return x;
-}
-
-__device__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int tile, int cap,
-                            const EmitScratch &sc, const sph_book &book)
-{
-    static_assert(R == 128 && kWave == 64, "two ballots cover a tile's rows");
-    static_assert(R / SPH_GROUP <= 8 && R <= 128, "a group descriptor packs k, a rank and a count into 8 bits each");
-    const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
-    const int wave = tid / kWave;
-
-    if (book.tile_nbr) { // the same pairs by stationary row: [k][row of the tile], coalesced
-        int32_t *dst = book.tile_nbr + (long)tile * KV * R;
-        for (int i = tid; i < KV * R; i += kThreads) {
-            const int k = i / R, r = i - k * R;
-            dst[i] = nbr[r * KV + k];
-        }
-    }
-    if (!book.grp_gather) return; // the caller keeps the pairs by row only: no groups, and no group counts either
-
-    // a wave takes every kWaves-th offset, eight of them per round with all their table reads in flight together
-    // (one LDS round trip per round instead of one per offset)
-    constexpr int kEmitBatch = 8;
-    for (int kb = wave; kb < KV; kb += kWaves * kEmitBatch) {
-        int v_lo[kEmitBatch], v_hi[kEmitBatch];
-#pragma unroll
-        for (int q = 0; q < kEmitBatch; q++) {
-            const int k = min(kb + q * kWaves, KV - 1);
-            v_lo[q] = nbr[lane * KV + k];
-            v_hi[q] = nbr[(kWave + lane) * KV + k];
-        }
-#pragma unroll
-        for (int q = 0; q < kEmitBatch; q++) {
-            const int k = min(kb + q * kWaves, KV - 1); // behind the last offset: the last one again, same values
-            {
-                const unsigned long long m0 = __ballot(v_lo[q] >= 0), m1 = __ballot(v_hi[q] >= 0);
-                const int c0 = __popcll(m0);
-                // set bits below this lane = the row's rank among the rows of its half
-                const int b0 = __builtin_amdgcn_mbcnt_hi((unsigned)(m0 >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m0, 0));
-                const int b1 = __builtin_amdgcn_mbcnt_hi((unsigned)(m1 >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m1, 0));
-                unsigned char *list = sc.sel + k * R;
-                if (v_lo[q] >= 0) list[b0] = (unsigned char)lane;
-                if (v_hi[q] >= 0) list[c0 + b1] = (unsigned char)(kWave + lane);
-                sc.cnt[k] = c0 + __popcll(m1); // every lane the same value
-            }
-        }
-    }
-    lds_barrier();
-    if (wave == 0) {
-        // exclusive scan of the per-offset group counts by one wave (KV <= 128: two passes)
-        int carry = 0;
-        for (int k0 = 0; k0 < KV; k0 += kWave) {
-            const int k = k0 + lane;
-            const int c = (k < KV) ? sc.cnt[k] : 0;
-            const int v = (c + SPH_GROUP - 1) / SPH_GROUP;
-            const int incl = wave_inclusive_sum(v);
-            if (k < KV) {
-                const int first = carry + incl - v;
-                sc.goff[k] = first;
-                for (int g = 0; g < v; g++) sc.ginfo[first + g] = k | (g * SPH_GROUP) << 8 | c << 16;
-            }
-            carry += __builtin_amdgcn_readlane(incl, kWave - 1);
-        }
-        if (lane == 0) {
-            sc.goff[KV] = carry;
-            book.tile_ngrp[tile] = carry;
-        }
-    }
-    lds_barrier();
-
-    for (int k = tid; k <= KV; k += kThreads)
-        book.tile_koff[(long)tile * (KV + 1) + k] = (uint16_t)sc.goff[k];
-    const int ngrp = sc.goff[KV];
-    const long gbase_tile = (long)tile * cap;
-    int32_t *out_gather = book.grp_gather + gbase_tile * SPH_GROUP, *out_owner = book.grp_owner + gbase_tile * SPH_GROUP;
-    // a thread's slots (slot, slot + kThreads, ...) four at a time: every step of the chain descriptor -> row ->
-    // table entry is one LDS round trip for the four together
-    constexpr int kEmitSlots = 4;
-    const int nslots = ngrp * SPH_GROUP;
-    for (int s0 = tid; s0 < nslots; s0 += kThreads * kEmitSlots) {
-        int info[kEmitSlots], row[kEmitSlots], gat[kEmitSlots];
-#pragma unroll
-        for (int q = 0; q < kEmitSlots; q++) info[q] = sc.ginfo[min(s0 + q * kThreads, nslots - 1) / SPH_GROUP];
-#pragma unroll
-        for (int q = 0; q < kEmitSlots; q++) {
-            // s0 and s0 + q * kThreads share their place in the group (kThreads is a multiple of the group size)
-            const int k = info[q] & 0xff, j = ((info[q] >> 8) & 0xff) + (tid & (SPH_GROUP - 1));
-            row[q] = j < (info[q] >> 16) ? sc.sel[k * R + j] : -1;
-        }
-#pragma unroll
-        for (int q = 0; q < kEmitSlots; q++) gat[q] = nbr[max(row[q], 0) * KV + (info[q] & 0xff)];
-#pragma unroll
-        for (int q = 0; q < kEmitSlots; q++) {
-            const int slot = s0 + q * kThreads;
-            if (slot < nslots) {
-                out_gather[slot] = row[q] >= 0 ? gat[q] : -1;
-                out_owner[slot] = row[q] >= 0 ? r0 + row[q] : -1;
-            }
-        }
-    }
-    for (int g = tid; g < ngrp; g += kThreads) book.grp_k[gbase_tile + g] = sc.ginfo[g] & 0xff;
-}
-
-// ---------------------------------------------------------------------------
-// Book builder by fiber join.  One block per tile of R stationary rows.
-//   1. map the tile's rows to their columns (block-wide search in q_ptr, then a
-//      walk over the covering columns);
-//   2. for every (row, k0, k1): locate the one column of the other grid that
-//      can pair with it and compare its fiber entries' S2 coordinate;
-//   3. emit_groups.
-// TRANSPOSED = false: stationary rows are outputs, x_d = o_d*s_d - p_d + k_d.
-// TRANSPOSED = true : stationary rows are inputs,  o_d = (x_d + p_d - k_d)/s_d.
-// ---------------------------------------------------------------------------
-struct BuildArgs {
-    const int32_t *q_idx, *q_ptr; // stationary side
-    const int32_t *p_idx, *p_ptr; // gathered side
-    int q_rows, p_rows;
-    int B;
-    Grid3 Q, P;
-    ConvParams cv;
-    int cap;
-    sph_book book;
-    // optional passenger: workgroups behind the tile workgroups pack a weight (total == 0: none)
-    SphPackJob pack;
-    int tile_blocks;
-    // gathered-side fibers are long (several entries on average) and their bins fit a 64-bit mask:
-    // join through per-column occupancy masks instead of walking a fiber once per row
-    int long_fibers;
-    FastDiv by_q1, by_q01; // division by Q.n1 and by Q.n0 * Q.n1
-};
-
-constexpr int kMaskCols = 32;  // distinct columns of a tile the mask join provides for
-constexpr int kMaskWalk = 16;  // fiber entries fetched together when a mask is built
-constexpr int kJoinItems = 5; // (row, k0, k1) items a thread joins per pass, all loads of a pass in flight together
-
+// Book builder: one workgroup per tile of R stationary rows (tile_table, then emit_groups); workgroups behind
+// the tiles' pack a weight.
 template <bool TRANSPOSED>
 __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
 {
-    extern __shared__ __attribute__((aligned(16))) int32_t s_nbr[]; // [R * KV]
-    __shared__ int s_col[R];
-    __shared__ int s_first[2 * kWaves], s_flag[2];
-
+    extern __shared__ __attribute__((aligned(16))) int32_t s_nbr[]; // [R * KV], emit scratch, masks of the mask join
     const int tid = threadIdx.x;
     if ((int)blockIdx.x >= a.tile_blocks) {
         // a weight rides along with the rule generation: the copy needs a launch of its own
@@ -320,250 +31,10 @@ __global__ __launch_bounds__(kThreads) void build_book_kernel(BuildArgs a)
     }
     const int tile = sph_xcd_tile(blockIdx.x, (a.q_rows + R - 1) / R);
     const int KV = a.cv.K0 * a.cv.K1 * a.cv.K2;
-    const int K01 = a.cv.K0 * a.cv.K1;
     const int r0 = tile * R;
     if (r0 >= a.q_rows) return; // grid is padded to a multiple of the XCD count
-    const int r1 = min(r0 + R, a.q_rows);
-    const int nrows = r1 - r0;
-    const int q_ncol = a.B * a.Q.n0 * a.Q.n1;
-
-    // the tile's own S2 coordinates do not depend on the column search: fetch them first.  A row belongs to
-    // the kThreads / R threads that share its number: each keeps the row's coordinates in registers.
-    static_assert(kThreads % R == 0, "a thread's items must share a row");
-    const int my_rl = tid & (R - 1);
-    const int my_zz = (my_rl < nrows) ? a.q_idx[r0 + my_rl] : 0;
-
-    // 1. rows -> columns.  The walk below tolerates starting early (columns before the
-    // tile hold none of its rows), so the search stops once the window is below one
-    // walk step: a single round of probes for grids of up to 131072 columns.
-    constexpr int kWalk = 2 * kThreads; // columns per walk step, two consecutive ones per thread
-    int c_first = block_upper_bound(a.q_ptr, q_ncol, r0, kWalk, s_first, [&]() {
-        for (int i = tid; i < R * KV / 4; i += kThreads) ((int4 *)s_nbr)[i] = make_int4(-1, -1, -1, -1); // R * KV is a multiple of 4
-        for (int i = tid; i < R; i += kThreads) s_col[i] = -1;
-    });
-    bool done = (c_first >= q_ncol);
-    for (int cb = c_first, step = 0; !done; cb += kWalk, step ^= 1) { // the steps alternate between two flags: one barrier each
-        const int last = min(cb + kWalk - 1, q_ncol - 1);
-        const int c = cb + 2 * tid;
-        if (c <= last) {
-            // q_ptr[c-1], q_ptr[c], q_ptr[c+1] bound the fibers of columns c and c+1
-            int p0 = c ? clampi(a.q_ptr[c - 1], 0, a.q_rows) : 0;
-            int p1 = clampi(a.q_ptr[c], 0, a.q_rows);
-            int p2 = (c + 1 <= last) ? clampi(a.q_ptr[c + 1], 0, a.q_rows) : p1;
-            if (p1 < p0) p1 = p0;
-            if (p2 < p1) p2 = p1;
-            for (int r = max(p0, r0); r < min(p1, r1); r++) s_col[r - r0] = c;
-            for (int r = max(p1, r0); r < min(p2, r1); r++) s_col[r - r0] = c + 1;
-            if (c == last || c + 1 == last) s_flag[step] = (p2 >= r1) || (last == q_ncol - 1);
-        }
-        lds_barrier();
-        done = s_flag[step] != 0;
-    }
-    // the row's column -> (batch, S0, S1), by every thread for its own row
-    const int my_c = my_rl < nrows ? s_col[my_rl] : -1;
-    const bool my_ok = my_c >= 0;
-    const int my_b = (int)div_by((uint32_t)max(my_c, 0), a.by_q01);
-    const int my_rem = max(my_c, 0) - my_b * (a.Q.n0 * a.Q.n1);
-    const int my_c0 = (int)div_by((uint32_t)my_rem, a.by_q1), my_c1 = my_rem - my_c0 * a.Q.n1;
-
-    // 2a. join through masks (long fibers).  The tile's rows share few columns, and every row of
-    // a column would walk the same K0*K1 fibers of the other grid: walk each (column, k0, k1)
-    // fiber once into a 64-bit occupancy mask, then every (row, k0, k1, k2) is a bit test and a
-    // popcount (position inside the sorted fiber).  A fiber that is not strictly ascending or
-    // leaves the 64 bins sends the whole tile to the general join below.
-    bool by_masks = false;
-    if (a.long_fibers) {
-        unsigned long long *s_cmask = (unsigned long long *)((char *)(s_nbr + R * KV) + emit_scratch_bytes(KV)); // [K01][ncols], ncols <= kMaskCols
-        int *s_cstart = (int *)(s_cmask + kMaskCols * K01);
-        __shared__ int s_b[R], s_c0[R], s_c1[R], s_z[R];
-        __shared__ int s_cj[R], s_rep[R], s_bad;
-        if (tid < R && my_ok) {
-            s_b[tid] = my_b;
-            s_c0[tid] = my_c0;
-            s_c1[tid] = my_c1;
-            s_z[tid] = my_zz;
-        }
-        __shared__ unsigned long long s_bal[R / kWave];
-        const int lane = tid & (kWave - 1), wave = tid / kWave;
-        if (tid == 0) s_bad = 0;
-        bool head = false;
-        if (tid < R) {
-            head = tid < nrows && s_col[tid] >= 0 && (tid == 0 || s_col[tid] != s_col[tid - 1]);
-            const unsigned long long bal = __ballot(head);
-            if (lane == 0) s_bal[wave] = bal;
-        }
-        lds_barrier();
-        int ncols = 0;
-        for (int w = 0; w < R / kWave; w++) ncols += __popcll(s_bal[w]);
-        if (tid < R) {
-            int incl = __popcll(s_bal[wave] & ((2ull << lane) - 1ull)); // heads at or before this row
-            for (int w = 0; w < wave; w++) incl += __popcll(s_bal[w]);
-            const int cj = (tid < nrows && s_col[tid] >= 0) ? incl - 1 : -1;
-            s_cj[tid] = cj;
-            if (head) s_rep[cj] = tid;
-        }
-        lds_barrier();
-        if (ncols > kMaskCols) ncols = 0; // short fibers after all: general join
-        for (int it = tid; it < ncols * K01; it += kThreads) {
-            const int k01 = it / ncols, cj = it - k01 * ncols;
-            const int rr = s_rep[cj];
-            const int k0 = k01 / a.cv.K1, k1 = k01 - k0 * a.cv.K1;
-            bool ok = true;
-            int y0, y1;
-            if (!TRANSPOSED) {
-                y0 = s_c0[rr] * a.cv.s0 - a.cv.p0 + k0;
-                y1 = s_c1[rr] * a.cv.s1 - a.cv.p1 + k1;
-            } else {
-                int t0 = s_c0[rr] + a.cv.p0 - k0, t1 = s_c1[rr] + a.cv.p1 - k1;
-                if (t0 < 0 || t1 < 0 || t0 % a.cv.s0 || t1 % a.cv.s1) ok = false;
-                y0 = t0 / a.cv.s0;
-                y1 = t1 / a.cv.s1;
-            }
-            if (y0 < 0 || y0 >= a.P.n0 || y1 < 0 || y1 >= a.P.n1) ok = false;
-            unsigned long long m = 0;
-            int st = 0;
-            if (ok) {
-                int e;
-                fiber_range(a.p_ptr, (s_b[rr] * a.P.n0 + y0) * a.P.n1 + y1, a.p_rows, st, e);
-                int prev = -1;
-                bool bad = false;
-                for (int e0 = st; e0 < e; e0 += kMaskWalk) {
-                    int v[kMaskWalk];
-#pragma unroll
-                    for (int q = 0; q < kMaskWalk; q++) v[q] = a.p_idx[min(e0 + q, e - 1)];
-#pragma unroll
-                    for (int q = 0; q < kMaskWalk; q++)
-                        if (e0 + q < e) {
-                            if ((unsigned)v[q] >= 64u || v[q] <= prev) bad = true;
-                            else m |= 1ull << v[q];
-                            prev = v[q];
-                        }
-                }
-                if (bad) s_bad = 1;
-            }
-            s_cmask[it] = m;
-            s_cstart[it] = st;
-        }
-        lds_barrier();
-        by_masks = s_bad == 0 && ncols > 0;
-        const bool pow2_s2 = (a.cv.s2 & (a.cv.s2 - 1)) == 0;
-        const int sh_s2 = __ffs(a.cv.s2) - 1;
-        if (by_masks) {
-            for (int it = tid; it < K01 * R; it += kThreads) {
-                const int rl = it & (R - 1), k01 = it / R;
-                const int cj = s_cj[rl];
-                if (cj < 0) continue;
-                const unsigned long long m = s_cmask[k01 * ncols + cj];
-                if (!m) continue;
-                const int st = s_cstart[k01 * ncols + cj], zz = s_z[rl];
-                for (int k2 = 0; k2 < a.cv.K2; k2++) {
-                    int v;
-                    if (!TRANSPOSED) {
-                        v = zz * a.cv.s2 - a.cv.p2 + k2;
-                    } else {
-                        const int t = zz + a.cv.p2 - k2;
-                        if (pow2_s2) { // uniform: strides 1, 2, 4, ... need no division
-                            if (t < 0 || (t & (a.cv.s2 - 1))) continue;
-                            v = t >> sh_s2;
-                        } else {
-                            if (t < 0 || t % a.cv.s2) continue;
-                            v = t / a.cv.s2;
-                        }
-                    }
-                    if ((unsigned)v < 64u && ((m >> v) & 1ull))
-                        s_nbr[rl * KV + k01 * a.cv.K2 + k2] = st + __popcll(m & ((1ull << v) - 1ull));
-                }
-            }
-        }
-    }
-
-    // 2. join.  item = (k01, row), consecutive lanes take consecutive rows.  Per pass a
-    // thread first issues the two fiber-bound loads of all its items, then the first
-    // three S2 coordinates of every fiber, and only then compares; longer fibers finish
-    // in a loop.
-    // kThreads is a multiple of R, so a thread meets the same row in every item: what depends on the row
-    // only is fetched from LDS and multiplied once, and an item costs a handful of integer operations
-    // (k0 = k01 / K1 by a 16-bit reciprocal, exact for the k01 < 256 that a kernel volume <= 128 allows)
-    const int my_a0 = TRANSPOSED ? my_c0 + a.cv.p0 : my_c0 * a.cv.s0 - a.cv.p0;
-    const int my_a1 = TRANSPOSED ? my_c1 + a.cv.p1 : my_c1 * a.cv.s1 - a.cv.p1;
-    const int my_col0 = my_b * a.P.n0;
-    const int my_slot = my_rl * KV;
-    const unsigned inv_k1 = (65536u + a.cv.K1 - 1) / a.cv.K1;
-    const bool unit_stride = a.cv.s0 == 1 && a.cv.s1 == 1;
-    const bool pow2_stride = (a.cv.s0 & (a.cv.s0 - 1)) == 0 && (a.cv.s1 & (a.cv.s1 - 1)) == 0;
-    const int sh_s0 = __ffs(a.cv.s0) - 1, sh_s1 = __ffs(a.cv.s1) - 1;
-    for (int base = 0; !by_masks && base < K01 * R; base += kThreads * kJoinItems) {
-        int ps[kJoinItems], len[kJoinItems], slot[kJoinItems];
-        int raw_e[kJoinItems], raw_s[kJoinItems];
-        bool ok[kJoinItems];
-#pragma unroll
-        for (int j = 0; j < kJoinItems; j++) {
-            const int k01 = (base + j * kThreads + tid) / R;
-            ok[j] = k01 < K01 && my_ok;
-            const int k0 = (int)(((unsigned)k01 * inv_k1) >> 16), k1 = k01 - k0 * a.cv.K1;
-            int y0, y1;
-            if (!TRANSPOSED) {
-                y0 = my_a0 + k0;
-                y1 = my_a1 + k1;
-            } else {
-                y0 = my_a0 - k0;
-                y1 = my_a1 - k1;
-                if (y0 < 0 || y1 < 0) ok[j] = false;
-                if (pow2_stride) { // uniform branches: shifts for strides 1, 2, 4, ..., divisions for the others
-                    if ((y0 & (a.cv.s0 - 1)) || (y1 & (a.cv.s1 - 1))) ok[j] = false;
-                    y0 >>= sh_s0;
-                    y1 >>= sh_s1;
-                } else if (!unit_stride) {
-                    if (y0 % a.cv.s0 || y1 % a.cv.s1) ok[j] = false;
-                    y0 /= a.cv.s0;
-                    y1 /= a.cv.s1;
-                }
-            }
-            if (y0 < 0 || y0 >= a.P.n0 || y1 < 0 || y1 >= a.P.n1) ok[j] = false;
-            const int pc = ok[j] ? (my_col0 + y0) * a.P.n1 + y1 : 0;
-            raw_e[j] = a.p_ptr[pc];
-            raw_s[j] = pc ? a.p_ptr[pc - 1] : 0;
-            slot[j] = my_slot + k01 * a.cv.K2;
-        }
-        int z0[kJoinItems], z1[kJoinItems], z2[kJoinItems];
-#pragma unroll
-        for (int j = 0; j < kJoinItems; j++) {
-            int e = clampi(raw_e[j], 0, a.p_rows), st = clampi(raw_s[j], 0, a.p_rows);
-            if (st > e) st = e;
-            ps[j] = st;
-            len[j] = ok[j] ? e - st : 0;
-            z0[j] = z1[j] = z2[j] = 0;
-            if (len[j] > 0) z0[j] = a.p_idx[st];
-            if (len[j] > 1) z1[j] = a.p_idx[st + 1];
-            if (len[j] > 2) z2[j] = a.p_idx[st + 2];
-        }
-#pragma unroll
-        for (int j = 0; j < kJoinItems; j++) {
-            // k2 of a gathered-side entry with S2 coordinate v: forward v is an input
-            // coordinate (k2 = v - (z*s2 - p2)), transposed v is an output coordinate
-            // (k2 = z + p2 - v*s2)
-            const int off = TRANSPOSED ? my_zz + a.cv.p2 : -(my_zz * a.cv.s2 - a.cv.p2);
-            const int mul = TRANSPOSED ? -a.cv.s2 : 1;
-            if (len[j] > 0) { int k2 = off + mul * z0[j]; if (k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j]; }
-            if (len[j] > 1) { int k2 = off + mul * z1[j]; if (k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j] + 1; }
-            if (len[j] > 2) { int k2 = off + mul * z2[j]; if (k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j] + 2; }
-            // longer fibers: four entries per round, their loads in flight together
-            for (int e = 3; e < len[j]; e += 4) {
-                int v[4];
-#pragma unroll
-                for (int q = 0; q < 4; q++) v[q] = a.p_idx[ps[j] + min(e + q, len[j] - 1)];
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const int k2 = off + mul * v[q];
-                    if (e + q < len[j] && k2 >= 0 && k2 < a.cv.K2) s_nbr[slot[j] + k2] = ps[j] + e + q;
-                }
-            }
-        }
-    }
-    lds_barrier();
-
-    // 3. compaction
-    emit_groups(s_nbr, nrows, r0, KV, tile, a.cap, emit_scratch_at(s_nbr + R * KV, KV), a.book);
+    tile_table<TRANSPOSED, true, kThreads>(a, tile, s_nbr, (char *)(s_nbr + R * KV) + emit_scratch_bytes(KV));
+    emit_groups<kThreads>(s_nbr, min(R, a.q_rows - r0), r0, KV, tile, a.cap, emit_scratch_at(s_nbr + R * KV, KV), a.book);
 }
 
 // Book builder from a global neighbour table nbr[rows, KV] (used when the rules
@@ -577,7 +48,7 @@ __global__ __launch_bounds__(kThreads) void book_from_nbr_kernel(const int32_t *
     const int nrows = min(R, rows - r0);
     for (int i = threadIdx.x; i < R * KV; i += kThreads) s_nbr[i] = i < nrows * KV ? nbr[(long)r0 * KV + i] : -1;
     lds_barrier();
-    emit_groups(s_nbr, nrows, r0, KV, tile, cap, emit_scratch_at(s_nbr + R * KV, KV), book);
+    emit_groups<kThreads>(s_nbr, nrows, r0, KV, tile, cap, emit_scratch_at(s_nbr + R * KV, KV), book);
 }
 
 // Kernel volumes above 96 need more than 48 KB of dynamic LDS for the neighbour table.
@@ -778,7 +249,8 @@ __global__ __launch_bounds__(kCountThreads) void outcoords_count_kernel(OutArgs 
 
 // oz_ptr holds the inclusive scan of the counts; one thread writes the bins of one column.
 __global__ __launch_bounds__(kThreads) void outcoords_fill_kernel(OutArgs a, const int32_t *oz_ptr, int32_t *oz_idx,
-                                                                  int out_rows, const unsigned long long *masks)
+                                                                  int out_rows, const unsigned long long *masks,
+                                                                  int32_t *row_cols)
 {
     const int ncol = a.B * a.O.n0 * a.O.n1;
     const int oc = blockIdx.x * kThreads + threadIdx.x;
@@ -794,7 +266,10 @@ __global__ __launch_bounds__(kThreads) void outcoords_fill_kernel(OutArgs a, con
         unsigned long long m = masks ? masks[(long)oc * nchunk + ch] : column_mask(a, b, o0, o1, ch, 0, 1);
         while (m) {
             int bit = __ffsll((long long)m) - 1;
-            if (pos < out_rows) oz_idx[pos] = ch * 64 + bit;
+            if (pos < out_rows) {
+                oz_idx[pos] = ch * 64 + bit;
+                if (row_cols) row_cols[pos] = oc;
+            }
             pos++;
             m &= m - 1;
         }
@@ -914,7 +389,7 @@ void sph_set_error(const char *fmt, ...)
 }
 
 SPH_EXPORT const char *sph_last_error(void) { return g_err; }
-SPH_EXPORT int sph_abi_version(void) { return 5; }
+SPH_EXPORT int sph_abi_version(void) { return 6; }
 SPH_EXPORT int sph_book_tiles(int rows) { return rows <= 0 ? 0 : sph_div_up(rows, R); }
 SPH_EXPORT int sph_book_cap(int KV) { return KV * (R / SPH_GROUP); }
 
@@ -937,7 +412,7 @@ SPH_EXPORT int sph_num_tiles(const sph_geom *g, int T0, int T1)
 
 static int rules_build(const char *who, const int32_t *z_idx, const int32_t *z_ptr, int in_rows, const int32_t *oz_idx,
                        const int32_t *oz_ptr, int out_rows, const sph_geom *g, int transposed, const sph_book *book,
-                       const SphPackJob *pack, void *stream)
+                       const int32_t *row_cols, const SphPackJob *pack, void *stream)
 {
     SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "%s: bad geometry (kernel volume <= %d)", who, SPH_MAX_KV);
     SPH_REQUIRE(book_ok(book), SPH_ERR_ARG, "%s: bad book", who);
@@ -958,6 +433,7 @@ static int rules_build(const char *who, const int32_t *z_idx, const int32_t *z_p
         a.p_idx = oz_idx; a.p_ptr = oz_ptr; a.p_rows = out_rows; a.P = O;
     }
     a.B = g->B;
+    a.q_rowcol = row_cols;
     a.cv = conv_params(g);
     a.by_q1 = fast_div((uint32_t)a.Q.n1);
     a.by_q01 = fast_div((uint32_t)a.Q.n0 * (uint32_t)a.Q.n1);
@@ -991,23 +467,25 @@ static int rules_build(const char *who, const int32_t *z_idx, const int32_t *z_p
 
 SPH_EXPORT int sph_rules_build(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
                                const int32_t *oz_idx, const int32_t *oz_ptr, int out_rows,
-                               const sph_geom *g, int transposed, const sph_book *book, void *stream)
+                               const sph_geom *g, int transposed, const sph_book *book,
+                               const int32_t *row_cols, void *stream)
 {
-    return rules_build("sph_rules_build", z_idx, z_ptr, in_rows, oz_idx, oz_ptr, out_rows, g, transposed, book, nullptr,
-                       stream);
+    return rules_build("sph_rules_build", z_idx, z_ptr, in_rows, oz_idx, oz_ptr, out_rows, g, transposed, book, row_cols,
+                       nullptr, stream);
 }
 
 SPH_EXPORT int sph_rules_build_pack(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
                                     const int32_t *oz_idx, const int32_t *oz_ptr, int out_rows,
                                     const sph_geom *g, int transposed, const sph_book *book,
+                                    const int32_t *row_cols,
                                     sph_dtype dt, const void *w, int KV, int kdim, int ndim, long stride_k,
                                     long stride_kk, long stride_n, void *packed, void *stream)
 {
     int rc = sph_pack_args_ok("sph_rules_build_pack", dt, w, packed, KV, kdim, ndim);
     if (rc) return rc;
     const SphPackJob p = sph_pack_job(dt, w, KV, kdim, ndim, stride_k, stride_kk, stride_n, packed);
-    return rules_build("sph_rules_build_pack", z_idx, z_ptr, in_rows, oz_idx, oz_ptr, out_rows, g, transposed, book, &p,
-                       stream);
+    return rules_build("sph_rules_build_pack", z_idx, z_ptr, in_rows, oz_idx, oz_ptr, out_rows, g, transposed, book,
+                       row_cols, &p, stream);
 }
 
 SPH_EXPORT int sph_outcoords_blocks(const sph_geom *g)
@@ -1138,7 +616,7 @@ SPH_EXPORT int sph_outcoords_count_static(const int32_t *z_idx, const int32_t *z
 
 SPH_EXPORT int sph_outcoords_fill(const int32_t *z_idx, const int32_t *z_ptr, int in_rows,
                                   const sph_geom *g, const int32_t *scratch, int32_t *oz_ptr,
-                                  int32_t *oz_idx, int out_rows, void *stream)
+                                  int32_t *oz_idx, int out_rows, int32_t *row_cols, void *stream)
 {
     SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_fill: bad geometry");
     SPH_REQUIRE(z_ptr && oz_ptr && scratch && out_rows >= 0 && (out_rows == 0 || oz_idx) &&
@@ -1146,7 +624,7 @@ SPH_EXPORT int sph_outcoords_fill(const int32_t *z_idx, const int32_t *z_ptr, in
     const int nb = sph_outcoords_blocks(g);
     hipLaunchKernelGGL(outcoords_fill_kernel, dim3(nb), dim3(kThreads), 0, (hipStream_t)stream,
                        out_args(z_idx, z_ptr, in_rows, g), (const int32_t *)oz_ptr, oz_idx, out_rows,
-                       (const unsigned long long *)outcoords_masks(g, (int32_t *)scratch));
+                       (const unsigned long long *)outcoords_masks(g, (int32_t *)scratch), row_cols);
     return sph_check_launch("sph_outcoords_fill");
 }
 
@@ -1211,4 +689,23 @@ SPH_EXPORT int sph_rules_from_padded(const int32_t *rules, const int32_t *rule_s
     hipLaunchKernelGGL(book_from_nbr_kernel, dim3(nt), dim3(kThreads), lds, st,
                        nbr, rows, KV, sph_book_cap(KV), *book);
     return sph_check_launch("sph_rules_from_padded");
+}
+
+// One thread per column writes the column's number to its rows.
+static __global__ void row_columns_kernel(const int32_t *z_ptr, int ncol, int rows, int32_t *row_cols)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= ncol) return;
+    int e = z_ptr[c], s = c ? z_ptr[c - 1] : 0;
+    e = e < rows ? e : rows;
+    for (int r = s < 0 ? 0 : s; r < e; r++) row_cols[r] = c;
+}
+
+SPH_EXPORT int sph_row_columns(const int32_t *z_ptr, int ncol, int rows, int32_t *row_cols, void *stream)
+{
+    SPH_REQUIRE(z_ptr && ncol > 0 && rows >= 0 && (rows == 0 || row_cols), SPH_ERR_ARG, "sph_row_columns: bad argument");
+    if (rows == 0) return SPH_OK;
+    hipLaunchKernelGGL(row_columns_kernel, dim3((unsigned)sph_div_up(ncol, 256)), dim3(256), 0, (hipStream_t)stream, z_ptr,
+                       ncol, rows, row_cols);
+    return sph_check_launch("sph_row_columns");
 }

@@ -26,6 +26,7 @@ class ConvFunction(torch.autograd.Function):
         ctx.tile_grid_shape = tile_grid_shape
         if packed is not None and weight.dtype != feature.dtype:
             packed = None                       # packed in the weight's type, the kernel needs the feature's
+        book.keep = True                        # backward walks the book
         return ext.rule_conv(feature, weight, book, None, outNNZ, packed=packed)
 
     @staticmethod

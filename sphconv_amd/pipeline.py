@@ -2,10 +2,13 @@
 stream of independent LiDAR scans, each scan on one of a few HIP streams.
 
 No reference counterpart (the reference launches everything on the legacy default
-stream, rule_conv.cu:139,333).  One 100k-voxel scan fills neither kernel's grid (a few
-hundred workgroups, one wave per SIMD), so the rule kernel of the next scan can run
-beside the convolution of the current one; the work per scan is unchanged.  All device
-memory (rule books, packed weights, outputs) is allocated once, per stream slot.
+stream, rule_conv.cu:139,333).  One 100k-voxel scan does not fill the chip, so the
+kernels of the next scan run beside those of the current one; the work per scan is
+unchanged.  All device memory (rule books, outputs) is allocated once, per stream slot;
+the weight is put in MFMA fragment order when the pipeline is made and again by
+``set_weight`` (a serving pipeline's weight changes when the model does, not per scan).
+A scan of up to RuleBook.FUSED_MAX_TILES tiles takes ONE launch (rules + forward,
+``sph_rules_conv``), a larger one two (``sph_rules_build``, ``sph_conv_apply``).
 """
 import ctypes as C
 from typing import List, Sequence, Tuple
@@ -13,7 +16,7 @@ from typing import List, Sequence, Tuple
 import torch
 
 from . import _lib as L
-from .rulebook import _Buffers, _check_index_tensors
+from .rulebook import RuleBook, _Buffers, _check_index_tensors, _row_cols_ptr
 
 
 class ScanPipeline:
@@ -26,7 +29,7 @@ class ScanPipeline:
     it must not overwrite them in place before the slot's scan has finished (``wait``)."""
 
     def __init__(self, weight: torch.Tensor, batch: int, shape: Sequence[int], kernel: Sequence[int] = (3, 3, 3),
-                 max_voxels: int = 1 << 18, streams: int = 3):
+                 max_voxels: int = 1 << 18, streams: int = 3, fused: bool = True):
         if weight.dim() == 5:
             weight = weight.reshape(-1, weight.shape[3], weight.shape[4])
         if weight.dim() != 3 or not weight.is_cuda:
@@ -50,21 +53,40 @@ class ScanPipeline:
         self._epi = L.Epilogue(None, None, 0)
         self._streams = [torch.cuda.Stream(device=dev) for _ in range(int(streams))]
         self._books = [_Buffers(self.max_voxels, self.kv, dev) for _ in self._streams]
-        self._packed = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in self._streams]
+        self._packed = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        self._packed_ready = torch.cuda.Event()
+        self.fused = bool(fused)
         self._out = [torch.empty((self.max_voxels, self.oc), dtype=self.weight.dtype, device=dev) for _ in self._streams]
         self._done = [torch.cuda.Event() for _ in self._streams]
         self._next = 0
         self._lib = lib
+        self.set_weight(self.weight)
+
+    def set_weight(self, weight: torch.Tensor):
+        """Takes (a new value of) the layer's weight: packs it on the caller's current stream; scans submitted
+        afterwards wait for the copy.  Scans still in flight may see either value: ``synchronize()`` first if
+        that matters."""
+        if weight.dim() == 5:
+            weight = weight.reshape(-1, weight.shape[3], weight.shape[4])
+        if tuple(weight.shape) != (self.kv, self.ic, self.oc) or weight.dtype != self.weight.dtype:
+            raise L.SphconvError("weight must stay [%d,%d,%d] %s" % (self.kv, self.ic, self.oc, self.weight.dtype))
+        self.weight = weight.detach().contiguous()
+        w = self.weight
+        L.check(self._lib.sph_weight_pack(self.dt, w.data_ptr(), self.kv, self.ic, self.oc, self.ic * self.oc, self.oc, 1,
+                                          self._packed.data_ptr(), L.stream()))
+        self._packed_ready.record(torch.cuda.current_stream())
+        self._packed_seen = [False] * len(self._streams)
 
     @property
     def streams(self) -> int:
         return len(self._streams)
 
     def submit(self, feature: torch.Tensor, z_idx: torch.Tensor, z_ptr: torch.Tensor,
-               wait_inputs: bool = True) -> Tuple[torch.Tensor, int]:
+               wait_inputs: bool = True, row_cols: torch.Tensor = None) -> Tuple[torch.Tensor, int]:
         """``wait_inputs=False`` skips making the slot's stream wait for the caller's current stream:
         only for inputs that are already complete (e.g. produced before a synchronisation, or on
-        ``stream_of(slot)`` itself)."""
+        ``stream_of(slot)`` itself).  ``row_cols`` (optional, int32 [n]): the column of every row
+        (``SparseConvTensor.row_cols``); saves the rule generation its search of ``z_ptr``."""
         n = int(z_idx.shape[0])
         if n > self.max_voxels:
             raise L.SphconvError("scan of %d voxels, pipeline sized for %d" % (n, self.max_voxels))
@@ -76,22 +98,30 @@ class ScanPipeline:
         side = self._streams[slot]
         if wait_inputs:
             side.wait_stream(torch.cuda.current_stream())   # the inputs were produced on the caller's stream
+        if not self._packed_seen[slot]:
+            side.wait_event(self._packed_ready)              # the packed weight was made on another stream
+            self._packed_seen[slot] = True
         # the kernels below read the inputs on the slot's stream: tell the caching allocator, so that a caller
         # who drops or rebinds them right after this call does not get their memory handed out again while
         # those kernels still run
-        for t in (feature, z_idx, z_ptr):
+        for t in (feature, z_idx, z_ptr) + ((row_cols,) if row_cols is not None else ()):
             t.record_stream(side)
         st = side.cuda_stream
         book = self._books[slot]
         book._struct.rows = n                                 # the slot's buffers hold up to max_voxels rows
-        lib, w = self._lib, self.weight
-        rc = lib.sph_rules_build_pack(z_idx.data_ptr(), z_ptr.data_ptr(), n, z_idx.data_ptr(), z_ptr.data_ptr(), n,
-                                      C.byref(self._geom), 0, C.byref(book._struct), self.dt, w.data_ptr(), self.kv,
-                                      self.ic, self.oc, self.ic * self.oc, self.oc, 1,
-                                      self._packed[slot].data_ptr(), st)
-        if rc == 0:
-            rc = lib.sph_conv_apply(self.dt, feature.data_ptr(), n, self.ic, self._packed[slot].data_ptr(), self.oc,
-                                    C.byref(book._struct), C.byref(self._epi), self._out[slot].data_ptr(), st)
+        lib = self._lib
+        hint = _row_cols_ptr(row_cols, n)
+        zi, zp = z_idx.data_ptr(), z_ptr.data_ptr()
+        rc = L.ERR_UNSUPPORTED
+        if self.fused and lib.sph_book_tiles(n) <= RuleBook.FUSED_MAX_TILES:
+            rc = lib.sph_rules_conv(zi, zp, n, zi, zp, n, C.byref(self._geom), C.byref(book._struct), 0, hint, self.dt,
+                                    feature.data_ptr(), self.ic, self._packed.data_ptr(), self.oc, C.byref(self._epi),
+                                    self._out[slot].data_ptr(), st)
+        if rc == L.ERR_UNSUPPORTED:
+            rc = lib.sph_rules_build(zi, zp, n, zi, zp, n, C.byref(self._geom), 0, C.byref(book._struct), hint, st)
+            if rc == 0:
+                rc = lib.sph_conv_apply(self.dt, feature.data_ptr(), n, self.ic, self._packed.data_ptr(), self.oc,
+                                        C.byref(book._struct), C.byref(self._epi), self._out[slot].data_ptr(), st)
         if rc:
             L.check(rc)
         self._done[slot].record(side)

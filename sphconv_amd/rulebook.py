@@ -82,6 +82,8 @@ class _Buffers:
         return int(((own >= 0) & used).sum().item())
 
 
+_NO_EPILOGUE = L.Epilogue(None, None, 0)
+
 # Estimated pairs per stationary row from which a book also keeps its pairs by row (and the
 # convolution walks that form).  float("inf") never does, 0 always.
 BY_ROW_MIN_PAIRS = 10.0
@@ -97,9 +99,12 @@ class RuleBook:
     """Pairs of one convolution geometry on one sparse tensor."""
 
     def __init__(self, z_idx, z_ptr, oz_idx, oz_ptr, batch, in_shape, out_shape, kernel, stride,
-                 padding, dilation, subm):
+                 padding, dilation, subm, row_cols=None, out_row_cols=None):
         self.z_idx, self.z_ptr = z_idx, z_ptr
         self.oz_idx, self.oz_ptr = oz_idx, oz_ptr
+        # optional: the column of every input / output row (what init_tensor and the output-coordinate kernels know
+        # when they write the rows); the rule kernel then need not search z_ptr for them
+        self.row_cols, self.out_row_cols = row_cols, out_row_cols
         self.batch = int(batch)
         self.in_shape = [int(v) for v in in_shape]
         self.out_shape = [int(v) for v in out_shape]
@@ -111,12 +116,28 @@ class RuleBook:
         self.kv = self.kernel[0] * self.kernel[1] * self.kernel[2]
         self.in_rows = int(z_idx.shape[0]) if z_idx is not None else 0
         self.out_rows = int(oz_idx.shape[0]) if oz_idx is not None else 0
-        self.fwd: Optional[_Buffers] = None
+        self._fwd: Optional[_Buffers] = None   # built on first use (see ``fwd``)
         self._bwd: Optional[_Buffers] = None
+        self.keep = True                       # a fused rules + forward launch also writes the book (``fused_forward``)
         self._padded = {}
         self._from_padded = None     # (rules, rule_size) when built from reference-format tensors
 
     # -- construction -----------------------------------------------------
+    @property
+    def fwd(self) -> _Buffers:
+        """The forward book (stationary on output rows); a book made with ``lazy=True`` is built here."""
+        if self._fwd is None:
+            self._fwd = self._build(False)
+        return self._fwd
+
+    @fwd.setter
+    def fwd(self, buf):
+        self._fwd = buf
+
+    @property
+    def built(self) -> bool:
+        return self._fwd is not None
+
     def geom(self) -> L.Geom:
         return L.make_geom(self.batch, self.in_shape, self.out_shape, self.kernel, self.stride,
                            self.padding, self.dilation)
@@ -158,10 +179,11 @@ class RuleBook:
         buf = _Buffers(rows, self.kv, self.z_ptr.device, by_row, groups)
         g, b = self.geom(), buf.struct()
         lib = L.lib()
+        hint = _row_cols_ptr(self.row_cols if transposed else self.out_row_cols, rows)
         if weight is None:
             rc = lib.sph_rules_build(self.z_idx.data_ptr(), self.z_ptr.data_ptr(), self.in_rows,
                                      self.oz_idx.data_ptr(), self.oz_ptr.data_ptr(), self.out_rows,
-                                     C.byref(g), int(transposed), C.byref(b), L.stream())
+                                     C.byref(g), int(transposed), C.byref(b), hint, L.stream())
             if rc:
                 L.check(rc)
             return buf
@@ -180,7 +202,7 @@ class RuleBook:
         packed = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
         rc = lib.sph_rules_build_pack(self.z_idx.data_ptr(), self.z_ptr.data_ptr(), self.in_rows,
                                       self.oz_idx.data_ptr(), self.oz_ptr.data_ptr(), self.out_rows,
-                                      C.byref(g), int(transposed), C.byref(b), dt, w.data_ptr(), kv, kdim, ndim,
+                                      C.byref(g), int(transposed), C.byref(b), hint, dt, w.data_ptr(), kv, kdim, ndim,
                                       wa * wb, skk, sn, packed.data_ptr(), L.stream())
         if rc:
             L.check(rc)
@@ -188,14 +210,20 @@ class RuleBook:
 
     @classmethod
     def build_subm(cls, z_idx, z_ptr, batch, shape, kernel, padding=None,
-                   dilation=(1, 1, 1), weight=None):
+                   dilation=(1, 1, 1), weight=None, row_cols=None, lazy=False):
         """Submanifold rules (replaces get_rules_subm, rules.cu:326-390): stride 1,
         outputs are the inputs; ``padding`` defaults to K//2 (conv.py:210).
         With ``weight`` [KV,iC,oC] returns ``(book, packed_weight)``: the layer's weight is
-        put in fragment order by the same kernel launch (pass it to ``rule_conv(..., packed=)``)."""
+        put in fragment order by the same kernel launch (pass it to ``rule_conv(..., packed=)``).
+        ``row_cols`` (optional, int32 [NNZ]): the column of every row (``SparseConvTensor.row_cols``).
+        ``lazy``: launch nothing yet; the pairs are generated by the first use -- by ``rule_conv`` in the same
+        launch as the convolution where the library has that kernel (:meth:`fused_forward`)."""
         _check_index_tensors(z_idx, z_ptr, batch, shape)
         pad = [int(k) // 2 for k in kernel] if padding is None else [int(v) for v in padding]
-        rb = cls(z_idx, z_ptr, z_idx, z_ptr, batch, shape, shape, kernel, (1, 1, 1), pad, dilation, True)
+        rb = cls(z_idx, z_ptr, z_idx, z_ptr, batch, shape, shape, kernel, (1, 1, 1), pad, dilation, True,
+                 row_cols, row_cols)
+        if lazy:
+            return rb
         if weight is None:
             rb.fwd = rb._build(False)
             return rb
@@ -234,7 +262,7 @@ class RuleBook:
 
     @classmethod
     def build(cls, z_idx, z_ptr, batch, in_shape, out_shape, kernel, stride, padding,
-              dilation=(1, 1, 1), weight=None, ahead=None):
+              dilation=(1, 1, 1), weight=None, ahead=None, row_cols=None, lazy=False):
         """Strided rules (replaces get_rules, rules.cu:405-486): output coordinates
         (oz_ptr inclusive scan, oz_idx ascending per column) and pairs.  One wait for the
         output row count, as in the reference (rules.cu:461): the count kernel writes it to pinned
@@ -273,12 +301,15 @@ class RuleBook:
                 raise
         out_rows = int(total[0])
         oz_idx = torch.empty(out_rows, dtype=torch.int32, device=dev)
+        out_cols = torch.empty(out_rows, dtype=torch.int32, device=dev)   # the output rows' columns, a by-product
         L.check(lib.sph_outcoords_fill(L.ptr(z_idx), L.ptr(z_ptr), n_in, C.byref(g), L.ptr(scratch),
-                                       L.ptr(oz_ptr), L.ptr(oz_idx), out_rows, L.stream()))
+                                       L.ptr(oz_ptr), L.ptr(oz_idx), out_rows, L.ptr(out_cols), L.stream()))
         if ahead is not None:
             _release_pinned_word(total)
         rb = cls(z_idx, z_ptr, oz_idx, oz_ptr, batch, in_shape, out_shape, kernel, stride, padding,
-                 dilation, False)
+                 dilation, False, row_cols, out_cols)
+        if lazy:                                     # output coordinates now, pairs with the first use
+            return rb
         if weight is None:
             rb.fwd = rb._build(False)
             return rb
@@ -302,6 +333,9 @@ class RuleBook:
         rb.kv = int(rules.shape[1])
         rb.in_rows, rb.out_rows = int(in_rows), int(out_rows)
         rb._bwd = None
+        rb._fwd = None
+        rb.keep = True
+        rb.row_cols = rb.out_row_cols = None
         rb._padded = {}
         rb._from_padded = (rules.contiguous(), rule_size.contiguous())
         rb.fwd = rb._convert(False)
@@ -319,6 +353,48 @@ class RuleBook:
                                               C.byref(b), L.stream()))
         return buf
 
+    # Tiles up to which one launch for rules + forward beats two (three workgroups of four waves, or four of two,
+    # per CU hold that many at once; beyond, the launch runs in rounds and the two kernels are as fast or faster:
+    # measured on the 64 x 2048 x 64 grid, 64 -> 64 fp16: 746 tiles 21.8 against 26.1 us, 937 tiles 29.3 / 32.0,
+    # 2457 tiles 68.6 / 66.9, 5957 tiles 140 / 142).
+    FUSED_MAX_TILES = 1024
+
+    def fused_forward(self, feature: torch.Tensor, packed: torch.Tensor, kdim: int, ndim: int, epilogue=None,
+                      out: Optional[torch.Tensor] = None, buffers: Optional[_Buffers] = None):
+        """Pairs and forward convolution of this (not yet built) book in ONE launch (``sph_rules_conv``): replaces
+        get_rules_subm / get_rules' pair half + rule_conv (rules.cu:326-486, rule_conv.cu:286-336) where the
+        reference launches three kernels.  Returns the output rows, or None when this layer is better served by
+        the two kernels (dense neighbourhoods that go by rows, more than FUSED_MAX_TILES tiles, shapes the
+        library's fused kernel does not take).  With ``self.keep`` the book is written too and the object counts
+        as built afterwards; without, only the output exists and a later use of the book generates it."""
+        if self._fwd is not None or self._from_padded is not None:
+            return None
+        lib = L.lib()
+        es = feature.element_size()
+        ntiles = lib.sph_book_tiles(self.out_rows)
+        if self.out_rows == 0 or ntiles > self.FUSED_MAX_TILES or self.kv > 32 or ndim > 64 \
+                or (kdim * es) % 16 or kdim * es > 128 or self._pairs_per_row(False) >= BY_ROW_MIN_PAIRS * BY_ROW_FORWARD_ONLY:
+            return None
+        if not feature.is_contiguous():
+            feature = feature.contiguous()
+        buf = buffers if buffers is not None else _Buffers(self.out_rows, self.kv, self.z_ptr.device)
+        if out is None:
+            out = torch.empty((self.out_rows, ndim), dtype=feature.dtype, device=feature.device)
+        g = self.geom()
+        epi = epilogue if epilogue is not None else _NO_EPILOGUE
+        rc = lib.sph_rules_conv(self.z_idx.data_ptr(), self.z_ptr.data_ptr(), self.in_rows, self.oz_idx.data_ptr(),
+                                self.oz_ptr.data_ptr(), self.out_rows, C.byref(g), C.byref(buf.struct()), int(self.keep),
+                                _row_cols_ptr(self.out_row_cols, self.out_rows), L.dtype_code(feature.dtype),
+                                feature.data_ptr(), int(kdim), packed.data_ptr(), int(ndim), C.byref(epi), out.data_ptr(),
+                                L.stream())
+        if rc == L.ERR_UNSUPPORTED:
+            return None
+        if rc:
+            L.check(rc)
+        if self.keep:
+            self._fwd = buf
+        return out
+
     # -- views ------------------------------------------------------------
     def grouped(self, transposed: bool = False) -> _Buffers:
         """The forward (or transposed) book with its groups, which wgrad, the padded tensors and the
@@ -329,7 +405,7 @@ class RuleBook:
             if transposed:
                 self._bwd = buf
             else:
-                self.fwd = buf
+                self._fwd = buf
         return buf
 
     def mirrored(self) -> bool:
@@ -421,6 +497,21 @@ def _pinned_word():
 def _release_pinned_word(word):
     if len(_PINNED_WORDS) < 64:
         _PINNED_WORDS.append(word)
+
+
+def _row_cols_ptr(row_cols, rows: int):
+    """Device pointer of a table of the rows' columns, or None when there is none (or it does not fit)."""
+    if row_cols is None or not row_cols.is_cuda or row_cols.dtype != torch.int32 or not row_cols.is_contiguous() \
+            or row_cols.dim() != 1 or row_cols.shape[0] != rows:
+        return None
+    return row_cols.data_ptr()
+
+
+def row_columns(z_ptr: torch.Tensor, rows: int) -> torch.Tensor:
+    """int32 [rows]: the column (index into the flattened ``z_ptr``) of every row."""
+    out = torch.empty(int(rows), dtype=torch.int32, device=z_ptr.device)
+    L.check(L.lib().sph_row_columns(L.ptr(z_ptr), z_ptr.numel(), int(rows), L.ptr(out), L.stream()))
+    return out
 
 
 def _check_index_tensors(z_idx, z_ptr, batch, shape):

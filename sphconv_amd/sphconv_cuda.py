@@ -30,24 +30,39 @@ MAX_TRAIN_CHANNELS = 128
 
 __version__ = "hip-gfx950"
 
-# Packed copies of weights seen while no gradient is being recorded (inference): one per (weight storage,
-# form), valid as long as the tensor object lives and its version counter, which every in-place update
-# bumps, has not moved.
+# Packed copies of weights, kept only for callers that ask for it (``cache=True``: modules in eval mode, under
+# ``torch.no_grad()``): one per (weight tensor, form), valid while the tensor object lives and its version
+# counter, storage address, shape and type have not moved.
 _PACKED_CACHE = {}
 
 
-def _packed_weight(weight: torch.Tensor, transpose: bool, reverse: bool = False) -> torch.Tensor:
+def invalidate_packed(weight: Optional[torch.Tensor] = None):
+    """Forgets the kept packed copies of ``weight`` (all of them when None).  Needed after an update the version
+    counter does not see: ``weight.data.mul_(2)`` or ``weight.data.copy_(...)`` change the values and leave
+    ``weight._version`` where it was."""
+    if weight is None:
+        _PACKED_CACHE.clear()
+        return
+    base = weight._base if weight._base is not None else weight
+    for key in [k for k in _PACKED_CACHE if k[0] == id(base)]:
+        _PACKED_CACHE.pop(key, None)
+
+
+def _packed_weight(weight: torch.Tensor, transpose: bool, reverse: bool = False, cache: bool = False) -> torch.Tensor:
     """weight [KV, a, b] -> fragment-ordered copy for the contraction over ``a``
     (``transpose``: over ``b``, i.e. with W[k]^T; ``reverse``: offsets in reverse order, W[KV-1-k]).
-    While gradients are being recorded the copy is made on every call (an optimiser step may follow);
-    under ``torch.no_grad()`` it is kept with the weight and reused until the weight changes."""
+    The copy is made on every call (a weight may have been updated in place) unless the caller passes
+    ``cache=True`` while no gradient is being recorded: then it is kept with the weight and reused until the
+    weight's version counter, address, shape or type change.  Updates through ``weight.data`` do not move the
+    version counter: call :func:`invalidate_packed` after them (modules: ``Convolution.invalidate_packed()``).
+    The kept copy belongs to the stream it was made on; other streams must order themselves behind it."""
     w = weight.detach()
     if not w.is_contiguous():
         w = w.contiguous()
     cache_key = None
-    if not torch.is_grad_enabled() and w.data_ptr() == weight.data_ptr():
+    if cache and not torch.is_grad_enabled() and w.data_ptr() == weight.data_ptr():
         base = weight._base if weight._base is not None else weight
-        cache_key = (id(base), bool(transpose), bool(reverse))
+        cache_key = (id(base), bool(transpose), bool(reverse), L.stream())
         state = (base._version, w.data_ptr(), tuple(w.shape), w.dtype)
         hit = _PACKED_CACHE.get(cache_key)
         if hit is not None and hit[0]() is base and hit[1] == state:
@@ -232,23 +247,32 @@ def _check_conv_args(feature, weight):
 
 def rule_conv(feature: torch.Tensor, weight: torch.Tensor, rules, ruleSize, outNNZ: int,
               scale: Optional[torch.Tensor] = None, shift: Optional[torch.Tensor] = None,
-              relu: bool = False, packed: Optional[torch.Tensor] = None) -> torch.Tensor:
+              relu: bool = False, packed: Optional[torch.Tensor] = None, cache_packed: bool = False) -> torch.Tensor:
     """rule_conv.cu:286-336: out[j] = sum over pairs (k,i,j) feature[i] @ weight[k].
     ``scale``/``shift`` (fp32 [oC]) and ``relu`` fuse y = relu(acc*scale + shift)
     into the store (no reference counterpart; default off).  ``packed``: the
     fragment-ordered copy of this very ``weight`` that ``RuleBook.build*(..., weight=)``
-    returned, which saves the packing launch."""
+    returned, which saves the packing launch; ``cache_packed``: keep the copy made here with the weight
+    (see :func:`_packed_weight`).  A RuleBook made with ``lazy=True`` gets its pairs generated by the same
+    launch that convolves them (``RuleBook.fused_forward``) where that is the faster way."""
     weight = _check_conv_args(feature, weight)
     book = _as_book(rules, ruleSize, feature.shape[0], int(outNNZ))
     if book.out_rows != int(outNNZ) or book.kv != weight.shape[0]:
         raise L.SphconvError("rules hold %d output rows / %d offsets, call says %d / %d"
                              % (book.out_rows, book.kv, int(outNNZ), weight.shape[0]))
     if packed is None:
-        packed = _packed_weight(weight, False)
+        packed = _packed_weight(weight, False, cache=cache_packed)
     elif packed.numel() != L.lib().sph_weight_packed_bytes(L.dtype_code(weight.dtype), weight.shape[0],
                                                            weight.shape[1], weight.shape[2]):
         raise L.SphconvError("packed weight of %d bytes does not belong to a weight of shape %s"
                              % (packed.numel(), tuple(weight.shape)))
+    if not book.built and feature.is_cuda and feature.shape[0] == book.in_rows:
+        epi = None
+        if scale is not None or shift is not None or relu:
+            epi = L.Epilogue(L.ptr(scale), L.ptr(shift), int(bool(relu)))
+        out = book.fused_forward(feature, packed, weight.shape[1], weight.shape[2], epi)
+        if out is not None:
+            return out
     return _apply(feature, packed, weight.shape[1], weight.shape[2], _conv_buffers(book, feature, weight, False),
                   scale, shift, relu)
 
@@ -275,8 +299,12 @@ def rule_conv_int8(feature: torch.Tensor, weight: torch.Tensor, scale: torch.Ten
     _check_conv_args(feature, weight)
     book = _as_book(rules, ruleSize, feature.shape[0], int(outNNZ))
     packed = _packed_weight(weight, False)
-    return _apply(feature, packed, weight.shape[1], weight.shape[2], _conv_buffers(book, feature, weight, False),
-                  scale.to(torch.float32).contiguous())
+    scale = scale.to(torch.float32).contiguous()
+    if not book.built and feature.is_cuda and feature.shape[0] == book.in_rows:
+        out = book.fused_forward(feature, packed, weight.shape[1], weight.shape[2], L.Epilogue(L.ptr(scale), None, 0))
+        if out is not None:
+            return out
+    return _apply(feature, packed, weight.shape[1], weight.shape[2], _conv_buffers(book, feature, weight, False), scale)
 
 
 def rule_conv_d_feature(feature: torch.Tensor, weight: torch.Tensor, rules, ruleSize,

@@ -23,8 +23,13 @@ class SparseConvTensor(SparseTensorBase):
 
     def __init__(self, raw_feature: torch.Tensor, spatial_shape_DWH: List[int], batch_size: int,
                  indices: Optional[torch.Tensor] = None, z_idx: Optional[torch.Tensor] = None,
-                 z_ptr: Optional[torch.Tensor] = None):
+                 z_ptr: Optional[torch.Tensor] = None, row_cols: Optional[torch.Tensor] = None):
         self.rule_cache = {}
+        # optional int32 [NNZ]: the column (index into the flattened z_ptr) of every row.  The reference's kernels
+        # get it from their launch geometry (one thread per column, rules.cu:256-259); here the rule kernel
+        # searches z_ptr for it unless the tensor brings it along.  Tensors made from COO indices and the outputs
+        # of convolutions carry it; ``with_row_cols()`` adds it to a tensor made from bare z_idx / z_ptr.
+        self.row_cols = row_cols
         self.requires_grad = False
         s0, s1, s2 = (int(v) for v in spatial_shape_DWH)
         if z_idx is not None and z_ptr is not None:
@@ -41,6 +46,15 @@ class SparseConvTensor(SparseTensorBase):
                          raw_feature.dtype, indices.dtype, None, None, None)
         self.feature, self.z_idx, self.z_ptr = InitTensorFunction.apply(
             raw_feature, indices, self.B, [self.D, self.W, self.H])
+        if self.z_ptr.is_cuda:
+            self.with_row_cols()
+
+    def with_row_cols(self):
+        """Computes ``row_cols`` from ``z_ptr`` (one small kernel) if the tensor does not have it yet."""
+        if self.row_cols is None and self.z_ptr is not None and self.z_ptr.is_cuda:
+            from .rulebook import row_columns
+            self.row_cols = row_columns(self.z_ptr, int(self.z_idx.shape[0]))
+        return self
 
     @property
     def shape(self):

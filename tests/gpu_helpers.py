@@ -15,6 +15,22 @@ def t(a, dtype=None):
     return x if dtype is None else x.to(dtype)
 
 
+def assert_same_conv(a, b):
+    """Two convolution kernels on the same pairs (grouped and by-row form, one launch and two) may add a row's
+    products in different orders: integer results are equal, floating-point results agree to the tolerance the
+    path promises (fp32 rtol 1e-5; fp16/bf16 rtol 1e-2, atol 1e-3).  Run-to-run determinism of ONE kernel is
+    asserted with torch.equal where it is tested."""
+    a = a if torch.is_tensor(a) else torch.as_tensor(a)
+    b = b if torch.is_tensor(b) else torch.as_tensor(b)
+    assert a.shape == b.shape and a.dtype == b.dtype
+    if not a.dtype.is_floating_point:
+        assert torch.equal(a, b)
+    elif a.dtype == torch.float32:
+        torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-5)   # atol: sums of products that cancel
+    else:
+        torch.testing.assert_close(a.float(), b.float(), rtol=1e-2, atol=1e-3)
+
+
 def book_triples(buf):
     """Decode one book on the host -> int64 array [P,3] of (k, gather, owner),
     sorted by (k, owner).  Also checks the structural invariants of the layout."""

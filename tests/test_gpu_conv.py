@@ -57,7 +57,7 @@ def test_fp32_forward_reference_lists(coords, args):
     # the reference-format entry: padded rules + rule_size through the same call
     rules, rule_size = book.padded((2, 2))
     out2 = ext.rule_conv(G.t(feat), G.t(w), rules, rule_size, book.out_rows).cpu().numpy()
-    assert np.array_equal(out, out2)
+    G.assert_same_conv(out, out2)      # by groups here, by rows above when that form is forced
     # and against torch's dense conv3d in float64
     dense = H.dense_from_rows(feat, case["sidx"], case["B"], case["shape"])
     y = H.dense_conv(dense, w.reshape(*a["kernel_size"], ic, oc), case["stride"], case["padding"], case["oshape"])
@@ -213,7 +213,7 @@ def test_fp32_backward(ic, oc, subm, kernel, stride, padding):
     if book.mirrored():   # dgrad ran on the forward book with mirrored offsets: same pairs, another order of summation
         np.testing.assert_allclose(d_feat2.cpu().numpy(), d_feat.cpu().numpy(), rtol=1e-5, atol=1e-5)
     else:
-        assert np.array_equal(d_feat2.cpu().numpy(), d_feat.cpu().numpy())
+        G.assert_same_conv(d_feat2, d_feat)
     assert np.array_equal(d_w2.cpu().numpy(), d_w.cpu().numpy())
     # float64 definition
     ref, _ = _f64_pair_sum(case, g.astype(np.float64), w.astype(np.float64), transposed=True)
@@ -499,7 +499,7 @@ def test_forward_only_book_builds_its_groups_on_demand(pair_form):
     assert book.fwd.groups == (pair_form == "groups")
     assert book.num_pairs() == ref_book.num_pairs()
     got = ext.rule_conv(feat, w, book, None, n, packed=packed)
-    assert torch.equal(got, want)
+    G.assert_same_conv(got, want)
     # 12 fp16 input channels are 24-byte rows: not a by-row call, needs the groups
     w12 = torch.tensor(_weights(rng, 27, 12, 16)).half().to(G.DEV)
     f12 = feat[:, :12].contiguous()
@@ -522,7 +522,8 @@ def test_forward_only_book_builds_its_groups_on_demand(pair_form):
                                                  (0.6, [24, 80, 16], 64, 32, torch.int8)])
 def test_by_row_equals_groups_on_large_grids(monkeypatch, p, shape, ic, oc, dtype):
     """More than 1024 tiles (one wave per tile in the by-row kernel), dense to sparse, rows of 32 and 64
-    bytes: same pairs, same summation order, so bit-identical to the grouped kernel, forward and dgrad."""
+    bytes: same pairs as the grouped kernel, forward and dgrad (int8 equal; floating point to the path's tolerance:
+    the two kernels add a row's products in different orders)."""
     from sphconv_amd import rulebook
     from sphconv_amd.rulebook import RuleBook
     rng = np.random.default_rng(int(p * 100) + ic)
@@ -552,10 +553,10 @@ def test_by_row_equals_groups_on_large_grids(monkeypatch, p, shape, ic, oc, dtyp
             g = torch.tensor(rng.standard_normal((n, oc)), dtype=torch.float32).to(dtype).to(G.DEV) if form == "groups" else g
             wt = w.permute(0, 2, 1).contiguous()
             out[form + "_d"] = ext.rule_conv_d_feature(g, wt, book, None, None, n)
-    assert torch.equal(out["groups"], out["by_row"])
+    G.assert_same_conv(out["groups"], out["by_row"])
     assert float(out["groups"].float().abs().mean()) > 0
     if dtype != torch.int8:
-        assert torch.equal(out["groups_d"], out["by_row_d"])
+        G.assert_same_conv(out["groups_d"], out["by_row_d"])
 
 
 @pytest.mark.parametrize("kernel,stride,padding,ic,oc,dtype", [([3, 3, 3], [2, 2, 2], [1, 1, 1], 32, 32, torch.float16),
@@ -565,7 +566,7 @@ def test_by_row_equals_groups_on_large_strided_grids(monkeypatch, kernel, stride
     """Strided layers with more than 1024 output tiles and 64-byte rows (the by-row kernel that stages the
     gathered rows in LDS, with footprints that do and do not fit its window, kernel volumes that are and
     are not a multiple of its phase of 9 offsets): forward on the book and dgrad on the transposed book
-    are bit-identical to the grouped kernels, and the forward result matches the oracle's."""
+    agree with the grouped kernels to the path's tolerance, and the forward result matches the oracle's."""
     from sphconv_amd import rulebook
     from sphconv_amd.rulebook import RuleBook
     rng = np.random.default_rng(ic + oc)
@@ -590,8 +591,8 @@ def test_by_row_equals_groups_on_large_strided_grids(monkeypatch, kernel, stride
         out[form] = ext.rule_conv(feat, w, book, None, m)
         g = torch.tensor(rng.standard_normal((m, oc)), dtype=torch.float32).to(dtype).to(G.DEV) if form == "groups" else g
         out[form + "_d"] = ext.rule_conv_d_feature(g, wt, book, None, None, n)
-    assert torch.equal(out["groups"], out["by_row"])
-    assert torch.equal(out["groups_d"], out["by_row_d"])
+    G.assert_same_conv(out["groups"], out["by_row"])
+    G.assert_same_conv(out["groups_d"], out["by_row_d"])
     ora = O.get_rules(z_idx, z_ptr, B, shape, oshape, kernel, stride, padding, n_max=512)
     oz_idx, oz_ptr, rules, rule_size, dropped = ora
     assert dropped == 0 and oz_idx.shape[0] == m
@@ -629,7 +630,8 @@ def test_forward_only_books_go_by_rows_from_a_lower_density(monkeypatch):
         assert book.fwd.tile_nbr is None and book.fwd.groups
     a = ext.rule_conv(feat, w, fwd_only, None, n, packed=packed)
     b = ext.rule_conv(feat, w, plain, None, n)
-    assert torch.equal(a, b) and float(a.float().abs().mean()) > 0
+    G.assert_same_conv(a, b)
+    assert float(a.float().abs().mean()) > 0
     sparse = rng.random((B, *shape)) < 0.2       # estimate 5.4: below both thresholds
     _, z_idx2, z_ptr2, _ = H.csr_from_indices(np.argwhere(sparse).astype(np.int32), B, shape)
     with torch.no_grad():

@@ -161,35 +161,50 @@ def test_real_scan_through_the_whole_path(subm, stride, padding):
 
 
 def test_scan_pipeline_matches_the_plain_path():
-    """ScanPipeline (scans in flight on several HIP streams) returns the bits of
-    get_rulebook_subm + rule_conv for every scan, whatever slot it lands in."""
+    """ScanPipeline (scans in flight on several HIP streams) returns what get_rulebook_subm + rule_conv return
+    for every scan, whatever slot it lands in: the same bits with two launches per scan, the same values to the
+    path's tolerance with one (another order of summation)."""
     from sphconv_amd import sphconv_cuda as ext
     from sphconv_amd.pipeline import ScanPipeline
     from sphconv_amd.rulebook import RuleBook
     B, shape, ic, oc = 2, [10, 24, 16], 16, 32
     rng = np.random.default_rng(3)
     w = G.t((rng.standard_normal((3, 3, 3, ic, oc)) * 0.1).astype(np.float32)).half()
-    pipe = ScanPipeline(w, B, shape, max_voxels=4096, streams=3)
-    assert pipe.streams == 3
-    scans = []
-    for s in range(7):                                     # more scans than slots, different sizes
-        idx, feat = _inputs(10 + s, B, shape, ic, p=0.1 + 0.05 * s)
-        x = sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx))
-        book = RuleBook.build_subm(x.z_idx, x.z_ptr, B, shape, [3, 3, 3])
-        want = ext.rule_conv(x.feature, w.view(27, ic, oc), book, None, x.feature.shape[0])
-        scans.append((x, want))
-    torch.cuda.synchronize()
-    pending = []
-    for i, (x, want) in enumerate(scans):
-        out, slot = pipe.submit(x.feature, x.z_idx, x.z_ptr)
-        pending.append((out, slot, want))
-        if len(pending) == pipe.streams:                   # read a slot before it is used again
-            o, sl, wnt = pending.pop(0)
-            pipe.wait(sl)
-            assert torch.equal(o, wnt)
-    pipe.synchronize()
-    for o, sl, wnt in pending:
-        assert torch.equal(o, wnt)
+    for fused in (True, False):
+        pipe = ScanPipeline(w, B, shape, max_voxels=4096, streams=3, fused=fused)
+        assert pipe.streams == 3
+        scans = []
+        for s in range(7):                                     # more scans than slots, different sizes
+            idx, feat = _inputs(10 + s, B, shape, ic, p=0.1 + 0.05 * s)
+            x = sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx))
+            book = RuleBook.build_subm(x.z_idx, x.z_ptr, B, shape, [3, 3, 3])
+            want = ext.rule_conv(x.feature, w.view(27, ic, oc), book, None, x.feature.shape[0])
+            scans.append((x, want))
+        torch.cuda.synchronize()
+
+        def same(o, wnt):
+            # two launches per scan: the very kernels of the plain path; one launch: the same pairs, added in another order
+            if fused:
+                G.assert_same_conv(o, wnt)
+            else:
+                assert torch.equal(o, wnt)
+
+        pending = []
+        for i, (x, want) in enumerate(scans):
+            out, slot = pipe.submit(x.feature, x.z_idx, x.z_ptr, row_cols=x.row_cols if i % 2 else None)
+            pending.append((out, slot, want))
+            if len(pending) == pipe.streams:                   # read a slot before it is used again
+                o, sl, wnt = pending.pop(0)
+                pipe.wait(sl)
+                same(o, wnt)
+        pipe.synchronize()
+        for o, sl, wnt in pending:
+            same(o, wnt)
+    # a new weight is taken by the scans submitted after it
+    pipe.set_weight(2 * w)
+    out, slot = pipe.submit(scans[0][0].feature, scans[0][0].z_idx, scans[0][0].z_ptr)
+    pipe.wait(slot)
+    torch.testing.assert_close(out.float(), 2 * scans[0][1].float(), rtol=1e-2, atol=2e-3)
     with pytest.raises(sphconv.SphconvError):
         big = torch.zeros((5000, ic), dtype=torch.float16, device=G.DEV)
         pipe.submit(big, torch.zeros(5000, dtype=torch.int32, device=G.DEV), scans[0][0].z_ptr)
@@ -322,9 +337,11 @@ def test_config4_encoder_full_size_layer_by_layer():
     assert [x.D, x.W, x.H] == [4, 128, 4] and x.feature.shape[1] == 64
 
 
-def test_packed_weight_is_kept_under_no_grad_and_follows_updates():
-    """Under torch.no_grad() the fragment-ordered copy of a weight is made once and reused until the weight's
-    version counter moves (an in-place update); while gradients are recorded it is made on every call."""
+def test_packed_weight_is_kept_only_on_request_and_follows_updates():
+    """The fragment-ordered copy of a weight is made on every call unless the caller asks to keep it (modules do
+    in eval mode under torch.no_grad()); a kept copy is reused until the weight's version counter moves (an
+    in-place update).  Updates through `.data` do not move the counter: they are seen at once by a module in
+    training mode, and by one in eval mode after `invalidate_packed()`."""
     from sphconv_amd import sphconv_cuda as ext
     B, shape = 1, [8, 16, 8]
     idx, feat = _inputs(3, B, shape, 16)
@@ -332,14 +349,28 @@ def test_packed_weight_is_kept_under_no_grad_and_follows_updates():
     x = sphconv.SparseConvTensor(G.t(feat).half(), shape, B, indices=G.t(idx))
     w = conv.weight.view(-1, 16, 32)
     with torch.no_grad():
-        p1 = ext._packed_weight(w, False)
-        assert ext._packed_weight(conv.weight.view(-1, 16, 32), False) is p1        # another view of the same parameter
-        assert ext._packed_weight(w, True) is not p1                                  # other form, other copy
+        assert ext._packed_weight(w, False) is not ext._packed_weight(w, False)     # not asked to keep: a copy per call
+        p1 = ext._packed_weight(w, False, cache=True)
+        assert ext._packed_weight(conv.weight.view(-1, 16, 32), False, cache=True) is p1   # another view of the parameter
+        assert ext._packed_weight(w, True, cache=True) is not p1                      # other form, other copy
+        conv.eval()
         y1 = conv(x).feature.clone()
         conv.weight.mul_(2.0)                                                         # bumps the version counter
-        p2 = ext._packed_weight(w, False)
+        p2 = ext._packed_weight(w, False, cache=True)
         assert p2 is not p1 and not torch.equal(p2, p1)
-        y2 = conv(x).feature
-    torch.testing.assert_close(y2.float(), 2 * y1.float(), rtol=2e-3, atol=2e-3)
+        y2 = conv(x).feature.clone()
+        torch.testing.assert_close(y2.float(), 2 * y1.float(), rtol=2e-3, atol=2e-3)
+        # through .data the version counter stays: eval mode keeps the old copy until it is told
+        v = conv.weight._version
+        conv.weight.data.mul_(2.0)
+        assert conv.weight._version == v
+        conv.invalidate_packed()
+        y3 = conv(x).feature.clone()
+        torch.testing.assert_close(y3.float(), 4 * y1.float(), rtol=2e-3, atol=4e-3)
+        # a module in training mode keeps nothing: the same kind of update is seen without being told
+        conv.train()
+        conv.weight.data.mul_(0.5)
+        y4 = conv(x).feature
+        torch.testing.assert_close(y4.float(), 2 * y1.float(), rtol=2e-3, atol=2e-3)
     with torch.enable_grad():
-        assert ext._packed_weight(w, False) is not ext._packed_weight(w, False)
+        assert ext._packed_weight(w, False, cache=True) is not ext._packed_weight(w, False, cache=True)

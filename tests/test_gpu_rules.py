@@ -345,5 +345,5 @@ def test_outcoords_scan_over_many_workgroups(shape, p):
         m = int(total[0])
         oz_idx = torch.full((max(m, 1),), -1, dtype=torch.int32, device="cuda:0")
         L.check(lib.sph_outcoords_fill(L.ptr(zi), L.ptr(zp), int(zi.shape[0]), C.byref(g), L.ptr(scratch),
-                                       L.ptr(oz_ptr), L.ptr(oz_idx), m, L.stream()))
+                                       L.ptr(oz_ptr), L.ptr(oz_idx), m, None, L.stream()))
         assert np.array_equal(oz_idx.cpu().numpy()[:m], np.nonzero(act.numpy())[3].astype(np.int32))

@@ -42,7 +42,7 @@ def _run(lib, zi, zp, B, shape, out_shape, static):
     m = int(total.item())
     oz_idx = torch.full((max(m, 1),), -1, dtype=torch.int32, device=G.DEV)
     L.check(lib.sph_outcoords_fill(L.ptr(zi), L.ptr(zp), n_in, C.byref(g), scratch_ptr, L.ptr(oz_ptr), L.ptr(oz_idx), m,
-                                   L.stream()))
+                                   None, L.stream()))
     torch.cuda.synchronize()
     return oz_ptr.cpu().numpy(), m, oz_idx.cpu().numpy()
 
