@@ -150,8 +150,9 @@ int sph_rules_build_pack(const int32_t *z_idx, const int32_t *z_ptr, int in_rows
  *     `scratch`: 8-byte aligned device memory of sph_outcoords_scratch_ints(g) int32, contents arbitrary;
  *     its first sph_outcoords_state_ints(g) entries hold the state of the scan across workgroups, which
  *     the count kernel clears for the scan behind it (calls that overlap on one scratch race).
- *     Behind the state, when O[2] <= 512, each column's 64-bit masks of active bins (one per 64 bins) are
- *     kept for step 2; deeper grids keep none and step 2 walks the fibers again.
+ *     Behind the state, when O[2] <= 512 and the masks of all columns take at most 128 MB, each column's
+ *     64-bit masks of active bins (one per 64 bins) are kept for step 2; deeper or larger grids keep none
+ *     and step 2 walks the fibers again.
  *  2. once the caller knows the total: sph_outcoords_fill, given the same scratch and oz_ptr, writes
  *     oz_idx (ascending within a column) and, when row_cols is not null, every output row's column
  *     (out_rows entries: the table sph_rules_build* takes for a layer that is stationary on these rows).

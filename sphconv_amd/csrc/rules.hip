@@ -168,7 +168,13 @@ __device__ __forceinline__ void column_masks(const OutArgs &a, int b, int o0, in
 }
 
 constexpr int kMaskChunks = 8;                   // chunks of 64 bins (O2 <= 512) up to which every column's masks are kept
+constexpr long kMaskWordsMax = 1L << 24;         // ... and 64-bit mask words (128 MB) up to which they are kept at all
 __host__ __device__ inline int mask_chunks(int O2) { return (O2 + 63) >> 6; }
+inline bool keeps_masks(const sph_geom *g)
+{
+    const int nchunk = mask_chunks(g->O[2]);
+    return nchunk <= kMaskChunks && (long)g->B * g->O[0] * g->O[1] * nchunk <= kMaskWordsMax;
+}
 
 constexpr int kColLanes = 16;                    // lanes that share one output column
 constexpr int kCountCols = 16;                   // output columns per workgroup of the count kernel
@@ -494,9 +500,10 @@ SPH_EXPORT int sph_outcoords_blocks(const sph_geom *g)
     return sph_div_up(g->B * g->O[0] * g->O[1], kThreads);
 }
 
-// int32 entries of the scratch the two calls share: the state of the scan across workgroups (two counters
-// and a 64-bit status word per workgroup of the count kernel) and, when a column's bins fit one 64-bit
-// mask, the masks behind it
+// int32 entries of the scratch the two calls share: the state of the scan of the counts (a ticket and one
+// 64-bit status word per tile of 2048 columns) and, behind it, every column's masks of active bins (one 64-bit
+// word per 64 bins) -- kept for grids of up to 512 bins and 128 MB of masks; deeper or larger grids keep none
+// and the fill kernel walks the fibers again
 SPH_EXPORT int sph_outcoords_state_ints(const sph_geom *g)
 {
     SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_state_ints: bad geometry");
@@ -508,14 +515,14 @@ SPH_EXPORT int sph_outcoords_scratch_ints(const sph_geom *g)
     SPH_REQUIRE(sph_geom_ok(g), SPH_ERR_ARG, "sph_outcoords_scratch_ints: bad geometry");
     const long ncol = (long)g->B * g->O[0] * g->O[1];
     const int nchunk = mask_chunks(g->O[2]);
-    const long n = scan_state_ints(ncol) + (nchunk <= kMaskChunks ? 2 * ncol * nchunk : 0);
+    const long n = scan_state_ints(ncol) + (keeps_masks(g) ? 2 * ncol * nchunk : 0);
     SPH_REQUIRE(n < 2147483647L, SPH_ERR_UNSUPPORTED, "sph_outcoords_scratch_ints: grid too large");
     return (int)n;
 }
 
 static unsigned long long *outcoords_masks(const sph_geom *g, int32_t *scratch)
 {
-    if (mask_chunks(g->O[2]) > kMaskChunks) return nullptr;
+    if (!keeps_masks(g)) return nullptr;
     return (unsigned long long *)(scratch + scan_state_ints((long)g->B * g->O[0] * g->O[1]));
 }
 

@@ -73,20 +73,17 @@ def xyz2RangeVoxel(points,
 
 
 class VoxelGenerator(object):
-    """data.py:12-26"""
+    """A fixed range-image geometry, applied to point clouds with ``generate`` (same constructor arguments and
+    attributes as data.py:12-26: resolutions, then ranges, then the log-depth switch)."""
+
+    _FIELDS = ("v_res", "h_res", "d_res", "v_range", "h_range", "d_range", "log")
 
     def __init__(self, v_res, h_res, d_res, v_range, h_range, d_range, log):
-        self.v_res = v_res
-        self.h_res = h_res
-        self.d_res = d_res
-        self.v_range = v_range
-        self.h_range = h_range
-        self.d_range = d_range
-        self.log = log
+        for name, value in zip(self._FIELDS, (v_res, h_res, d_res, v_range, h_range, d_range, log)):
+            setattr(self, name, value)
 
     def generate(self, points):
-        return xyz2RangeVoxel(points, self.v_res, self.h_res, self.d_res,
-                              self.v_range, self.h_range, self.d_range, self.log)
+        return xyz2RangeVoxel(points, *(getattr(self, name) for name in self._FIELDS))
 
 
 def merge_rangevoxel_batch(voxel_list: List[RangeVoxel]) -> RangeVoxel:

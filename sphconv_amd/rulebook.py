@@ -467,9 +467,20 @@ def _workspace_key(dev):
     return (index, torch.cuda.current_stream(index).cuda_stream)
 
 
+# The scratch holds 8 bytes per output column and 64 bins (up to 128 MB, see sph_outcoords_count): it scales with
+# the dense column grid, not with the number of voxels.  Up to this many int32 entries it is kept per (device,
+# stream) between calls; a larger one belongs to its call and goes back to the allocator with it.
+_WORKSPACE_KEEP_INTS = 1 << 24      # 64 MB
+
+
 def _outcoords_workspace(dev, nints: int):
     key = _workspace_key(dev)
     ws = _WORKSPACES.get(key)
+    if nints > _WORKSPACE_KEEP_INTS:
+        total = ws[1] if ws is not None else torch.zeros(1, dtype=torch.int32).pin_memory()
+        if ws is None:
+            _WORKSPACES[key] = (torch.empty(1 << 16, dtype=torch.int32, device=dev), total)
+        return torch.empty(nints + (nints & 1), dtype=torch.int32, device=dev), total
     if ws is None or ws[0].numel() < nints:
         scratch = torch.empty(max(nints + (nints & 1), 1 << 16), dtype=torch.int32, device=dev)
         total = ws[1] if ws is not None else torch.zeros(1, dtype=torch.int32).pin_memory()

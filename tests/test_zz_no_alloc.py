@@ -61,6 +61,36 @@ def test_static_scratch_matches_caller_scratch_twice():
         assert (got[2][:got[1]] >= 0).all()
 
 
+def test_static_scratch_allocates_nothing_and_is_one_array():
+    """What the entry point is for: between two calls the device's free memory does not move (no allocation, no
+    free, in the library or through torch), and every call names the same array."""
+    lib = L.lib()
+    zi, zp, out_shape = _case(4, 2, [32, 96, 24], 0.1)
+    B, shape = 2, [32, 96, 24]
+    g = L.make_geom(B, shape, out_shape, [3, 3, 3], [2, 2, 2], [1, 1, 1], [1, 1, 1])
+    oz_ptr = torch.empty((B, out_shape[0], out_shape[1]), dtype=torch.int32, device=G.DEV)
+    total = torch.empty((1,), dtype=torch.int32, device=G.DEV)
+    ptrs = []
+
+    def call():
+        sp = C.c_void_p()
+        L.check(lib.sph_outcoords_count_static(L.ptr(zi), L.ptr(zp), int(zi.shape[0]), C.byref(g), L.ptr(oz_ptr),
+                                               L.ptr(total), C.byref(sp), L.stream()))
+        ptrs.append(sp.value)
+
+    call()                                  # the first call on a device looks the array's address up
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    reserved0 = torch.cuda.memory_reserved()
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0 and torch.cuda.memory_reserved() == reserved0
+    assert len(set(ptrs)) == 1 and ptrs[0]
+    assert int(total.item()) > 0
+
+
 def test_static_scratch_rejects_grids_beyond_its_size():
     lib = L.lib()
     limit = L.STATIC_MAX_COLUMNS
