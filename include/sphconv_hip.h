@@ -228,14 +228,17 @@ int sph_conv_apply(sph_dtype dt, const void *feature, int feature_rows, int kdim
 /* get_rules_subm / get_rules' pair half (rules.cu:326-390, 445-485) and rule_conv (rule_conv.cu:286-336) of ONE
  * layer in ONE launch: every workgroup builds its tile's pairs in LDS as sph_rules_build does and convolves them
  * at once as sph_conv_apply does; `out` [out_rows, ndim] is fully overwritten.  Arguments as for sph_rules_build
- * (transposed == 0) and sph_conv_apply.  `book` must provide all group arrays: with write_book != 0 the book is
- * filled as sph_rules_build fills it (for layers that share it through an indice_key, or for a backward pass);
- * with write_book == 0 only tiles whose groups do not fit the workgroup's LDS (more than 64 groups) use their
- * part of it, and its contents are unspecified afterwards.  Returns SPH_ERR_UNSUPPORTED (nothing launched) for
+ * (transposed == 0) and sph_conv_apply.  `book` must provide all group arrays: with SPH_FUSED_WRITE_BOOK in
+ * `flags` the book is filled as sph_rules_build fills it (for layers that share it through an indice_key, or for
+ * a backward pass); without it only tiles whose groups do not fit the workgroup's LDS (more than 64 groups) use
+ * their part of it, and its contents are unspecified afterwards.  SPH_FUSED_IN_FLIGHT says that the caller keeps
+ * several scans in flight on streams of their own: the launch then uses two-wave workgroups, four of which fit a
+ * CU where three four-wave ones do -- a lone scan takes about a tenth longer, a stream of scans a tenth less.  Returns SPH_ERR_UNSUPPORTED (nothing launched) for
  * shapes the fused kernel does not take -- rows that are not 16-byte multiples of up to 128 bytes, more than 64
  * output channels, more than 32 kernel offsets: call sph_rules_build + sph_conv_apply then. */
+enum { SPH_FUSED_WRITE_BOOK = 1, SPH_FUSED_IN_FLIGHT = 2 };
 int sph_rules_conv(const int32_t *z_idx, const int32_t *z_ptr, int in_rows, const int32_t *oz_idx,
-                   const int32_t *oz_ptr, int out_rows, const sph_geom *g, const sph_book *book, int write_book,
+                   const int32_t *oz_ptr, int out_rows, const sph_geom *g, const sph_book *book, int flags,
                    const int32_t *row_cols, sph_dtype dt, const void *feature, int kdim, const void *packed_w,
                    int ndim, const sph_epilogue *epi, void *out, void *stream);
 

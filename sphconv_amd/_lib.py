@@ -19,6 +19,7 @@ STATIC_MAX_COLUMNS = 1 << 20     # SPH_STATIC_MAX_COLUMNS of the header
 
 F32, F16, BF16, I8 = 0, 1, 2, 3
 ERR_ARG, ERR_UNSUPPORTED, ERR_LAUNCH = -1, -2, -3      # sph_status
+FUSED_WRITE_BOOK, FUSED_IN_FLIGHT = 1, 2               # flags of sph_rules_conv
 _DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.int8: I8}
 
 

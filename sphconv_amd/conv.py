@@ -105,7 +105,7 @@ class Conv3d(Convolution):
         return RuleBook.count_ahead(input.z_idx, input.z_ptr, input.B, in_shape, out_shape, self.kernel_size,
                                     self.stride, self.padding, self.dilation)
 
-    def _rules(self, input: SparseConvTensor, out_shape, ahead=None, keep: bool = True):
+    def _rules(self, input: SparseConvTensor, out_shape, ahead=None, keep: bool = True, training: bool = True):
         """Rule book of this layer on ``input``, shared through ``rule_cache`` when an
         ``indice_key`` is set (conv.py:159-177).  A book that is not cached yet is returned unbuilt (for a strided
         layer with its output coordinates): ``rule_conv`` generates its pairs in the launch that convolves them
@@ -124,6 +124,8 @@ class Conv3d(Convolution):
                                   self.kernel_size, self.stride, self.padding, self.dilation, ahead=ahead,
                                   row_cols=row_cols, lazy=True)
         book.keep = bool(keep)
+        if not training:
+            book.forward_only = (self.in_channels, self.out_channels, input.feature.element_size())
         entry = (book.oz_idx, book.oz_ptr, book, None, get_tile_grid_shape(out_shape, self.tile_size))
         if self.indice_key is not None:
             input.rule_cache[self.indice_key] = entry
@@ -142,7 +144,7 @@ class Conv3d(Convolution):
         weight = self.weight.view(-1, self.in_channels, self.out_channels)
         training = torch.is_grad_enabled() and (weight.requires_grad or input.feature.requires_grad)
         oz_idx, oz_ptr, book, rule_size, tile_grid_shape = self._rules(
-            input, out_shape, ahead, keep=training or self.indice_key is not None)
+            input, out_shape, ahead, keep=training or self.indice_key is not None, training=training)
         self.rule_book = book if isinstance(book, RuleBook) else None
         if epilogue is not None:
             if training:

@@ -27,6 +27,7 @@ struct FusedArgs {
     ConvArgs c;
     int nwtot;      // 16-column tiles of the output, padded to 1, 2 or 4
     int write_book; // also store the tile's groups (and the by-row table, if the book has one)
+    int small_wg;   // two-wave workgroups (four fit a CU) whatever the tile count: for callers with scans in flight
 };
 
 inline size_t fused_region_a(int KV, int nwtot)
@@ -148,7 +149,7 @@ int launch_fused(const FusedArgs &fa, int ntiles, hipStream_t st)
 {
     // three workgroups of 256 threads per CU hold 768 tiles at once, four of 128 threads 1024 (and fp32 rows of 128
     // bytes into 64 columns do not fit the registers three workgroups leave a wave)
-    if (ntiles > 768 || (DT == SPH_F32 && NS == 2 && CT == 4)) return launch_fused_nt<DT, NS, CT, MASKED, 128>(fa, ntiles, st);
+    if (fa.small_wg || ntiles > 768 || (DT == SPH_F32 && NS == 2 && CT == 4)) return launch_fused_nt<DT, NS, CT, MASKED, 128>(fa, ntiles, st);
     return launch_fused_nt<DT, NS, CT, MASKED, 256>(fa, ntiles, st);
 }
 
@@ -180,7 +181,7 @@ int launch_fused_ns(const FusedArgs &fa, int ntiles, hipStream_t st)
 
 
 SPH_EXPORT int sph_rules_conv(const int32_t *z_idx, const int32_t *z_ptr, int in_rows, const int32_t *oz_idx,
-                              const int32_t *oz_ptr, int out_rows, const sph_geom *g, const sph_book *book, int write_book,
+                              const int32_t *oz_ptr, int out_rows, const sph_geom *g, const sph_book *book, int flags,
                               const int32_t *row_cols, sph_dtype dt, const void *feature, int kdim, const void *packed_w,
                               int ndim, const sph_epilogue *epi, void *out, void *stream)
 {
@@ -218,7 +219,8 @@ SPH_EXPORT int sph_rules_conv(const int32_t *z_idx, const int32_t *z_ptr, int in
     a.aligned_in = (a.row_bytes % 16 == 0) && ((uintptr_t)feature % 16 == 0);
     a.aligned_out = ((ndim * es) % 16 == 0) && ((uintptr_t)out % 16 == 0);
     fa.nwtot = sph_pad_waves(ndim);
-    fa.write_book = write_book != 0;
+    fa.write_book = (flags & SPH_FUSED_WRITE_BOOK) != 0;
+    fa.small_wg = (flags & SPH_FUSED_IN_FLIGHT) != 0;
     // what this kernel takes: whole 16-byte chunks of up to 128 bytes per row (with 256-byte rows the loop does not
     // fit the registers that three workgroups per CU leave a wave), up to 64 output columns, arrays below 2 GiB,
     // and a table of KV offsets per row that fits the accumulators' LDS

@@ -114,7 +114,8 @@ class ScanPipeline:
         zi, zp = z_idx.data_ptr(), z_ptr.data_ptr()
         rc = L.ERR_UNSUPPORTED
         if self.fused and lib.sph_book_tiles(n) <= RuleBook.FUSED_MAX_TILES:
-            rc = lib.sph_rules_conv(zi, zp, n, zi, zp, n, C.byref(self._geom), C.byref(book._struct), 0, hint, self.dt,
+            rc = lib.sph_rules_conv(zi, zp, n, zi, zp, n, C.byref(self._geom), C.byref(book._struct),
+                                    L.FUSED_IN_FLIGHT if len(self._streams) >= 3 else 0, hint, self.dt,
                                     feature.data_ptr(), self.ic, self._packed.data_ptr(), self.oc, C.byref(self._epi),
                                     self._out[slot].data_ptr(), st)
         if rc == L.ERR_UNSUPPORTED:

@@ -119,6 +119,9 @@ class RuleBook:
         self._fwd: Optional[_Buffers] = None   # built on first use (see ``fwd``)
         self._bwd: Optional[_Buffers] = None
         self.keep = True                       # a fused rules + forward launch also writes the book (``fused_forward``)
+        # (input channels, output channels, element size) of the forward pass a lazy book is made for, when no
+        # gradient will be asked of it: lets a book that goes by rows leave its groups out (see ``_build``)
+        self.forward_only: Optional[tuple] = None
         self._padded = {}
         self._from_padded = None     # (rules, rule_size) when built from reference-format tensors
 
@@ -157,8 +160,10 @@ class RuleBook:
         to 128 bytes, 16-byte multiples out, a table that fits LDS): the conditions of the library."""
         kv, wa, wb = weight.shape
         kdim, ndim = (wb, wa) if weight_transposed else (wa, wb)
-        es = weight.element_size()
-        return (kdim * es) % 16 == 0 and kdim * es <= 128 and (ndim * es) % 16 == 0 and kv * L.TILE_ROWS * 4 <= 48 * 1024
+        return self._rows_kernel_takes_shape(kdim, ndim, weight.element_size())
+
+    def _rows_kernel_takes_shape(self, kdim: int, ndim: int, es: int) -> bool:
+        return (kdim * es) % 16 == 0 and kdim * es <= 128 and (ndim * es) % 16 == 0 and self.kv * L.TILE_ROWS * 4 <= 48 * 1024
 
     def _build(self, transposed: bool, weight=None, weight_transposed: bool = False, groups: Optional[bool] = None):
         """Launches the rule kernel.  With ``weight`` [KV,a,b] its fragment-ordered copy (what
@@ -173,6 +178,8 @@ class RuleBook:
         if groups is None:
             forward_only = (weight is not None and not torch.is_grad_enabled() and weight.dim() == 3
                             and self._rows_kernel_takes(weight, weight_transposed))
+            if weight is None and not transposed and self.forward_only is not None and not torch.is_grad_enabled():
+                forward_only = self._rows_kernel_takes_shape(*self.forward_only)
             if forward_only:
                 by_row = est >= BY_ROW_MIN_PAIRS * BY_ROW_FORWARD_ONLY
             groups = not (by_row and forward_only)
@@ -335,6 +342,7 @@ class RuleBook:
         rb._bwd = None
         rb._fwd = None
         rb.keep = True
+        rb.forward_only = None
         rb.row_cols = rb.out_row_cols = None
         rb._padded = {}
         rb._from_padded = (rules.contiguous(), rule_size.contiguous())

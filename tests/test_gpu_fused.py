@@ -87,13 +87,13 @@ def test_one_launch_matches_the_oracle(subm, kernel, stride, padding, p, ic, oc,
     cols = row_columns(book.oz_ptr, m)
     tri = G.oracle_triples(rules, rule_size)
     for hint in (None, cols):
-        for write_book in (0, 1):
-            out, buf = _fused(case, feat.to(G.DEV), w.to(G.DEV), write_book, hint)
+        for flags in (0, L.FUSED_WRITE_BOOK, L.FUSED_IN_FLIGHT, L.FUSED_WRITE_BOOK | L.FUSED_IN_FLIGHT):
+            out, buf = _fused(case, feat.to(G.DEV), w.to(G.DEV), flags, hint)
             _check_out(out, want, dtype)
-            if write_book:
+            if flags & L.FUSED_WRITE_BOOK:
                 assert np.array_equal(G.book_triples(buf), tri)
     # twice the same call: the same bits
-    again, _ = _fused(case, feat.to(G.DEV), w.to(G.DEV), 0, cols)
+    again, _ = _fused(case, feat.to(G.DEV), w.to(G.DEV), L.FUSED_WRITE_BOOK | L.FUSED_IN_FLIGHT, cols)
     assert torch.equal(again, out)
 
 
