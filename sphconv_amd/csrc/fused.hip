@@ -64,39 +64,107 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(NT == 256 ? 
     unsigned char *m_own = (unsigned char *)(m_gat + kFusedGroups * SPH_GROUP);
     unsigned char *m_gk = m_own + kFusedGroups * SPH_GROUP;
     __shared__ unsigned long long s_cov[2];
+    __shared__ int s_cnt[32];
 
-    // 1. the tile's pairs: table, then lists and group descriptors
+    // region B starts as "no pair anywhere": the direct compaction below writes the slots that hold one
+    for (int i = tid; i < kFusedGroups * SPH_GROUP / 4; i += NT) ((int4v *)m_gat)[i] = int4v{-1, -1, -1, -1};
+
+    // 1. the tile's pairs: the table of (row, offset) -> gathered row
     tile_table<false, false, NT>(b, tile, s_nbr, nullptr);
     // The groups of the middle offset (in a submanifold layer: every row's pair with itself, a run of eight full
     // groups) go to the waves that would otherwise wait, and are the first the tile is given: stored, not added.
     // The compact arrays keep them behind the other groups.
     const int kc = KV / 2;
-    const int ngrp = emit_lists<NT>(s_nbr, KV, sc, kc);
-    const bool fits = ngrp <= kFusedGroups;
-    const int gc_lo = sc.goff[kc], nc = sc.goff[kc + 1] - gc_lo;
-    const int n0 = ngrp - nc;
-    if (fa.write_book && b.book.tile_nbr) emit_nbr_store(s_nbr, KV, tile, b.book, tid, NT);
-    if (fa.write_book || !fits) emit_store(s_nbr, r0, KV, tile, b.cap, sc, b.book, tid, NT);
-    if (fits) {
-        // one thread per slot: descriptor -> row -> table entry, as the store to the book does
-        for (int s = tid; s < ngrp * SPH_GROUP; s += NT) {
-            const int g = s / SPH_GROUP;
-            const int info = sc.ginfo[g];
-            const int k = info & 0xff, j = ((info >> 8) & 0xff) + (s & (SPH_GROUP - 1));
-            const int row = j < (info >> 16) ? sc.sel[k * R + j] : -1;
-            const int gpos = g < gc_lo ? g : (g < gc_lo + nc ? n0 + (g - gc_lo) : g - nc);
-            const int d = gpos * SPH_GROUP + (s & (SPH_GROUP - 1));
-            m_gat[d] = row >= 0 ? s_nbr[row * KV + k] : -1;
-            m_own[d] = (unsigned char)(row >= 0 ? row : 0);
-            if ((s & (SPH_GROUP - 1)) == 0) m_gk[gpos] = (unsigned char)k;
+    int ngrp = 0, n0 = 0;
+    bool fits = false;
+    if (!fa.write_book) {
+        // Nobody wants the book: the groups go from the table straight to region B.  A wave takes the offsets
+        // wave, wave + NW, ...: the table's column of an offset stays in two registers per lane (rows lane and
+        // lane + 64), two ballots count its pairs; behind one barrier every wave knows all counts, hence where an
+        // offset's groups start, and a row's rank in its offset's list (the bits below it in the ballots) is its
+        // slot.  Rows ascending inside an offset, offsets ascending, the middle offset last: the order of the lists
+        // that emit_lists makes, without the lists.
+        constexpr int KPW = (32 + NW - 1) / NW; // KV <= 32
+        int e_lo[KPW], e_hi[KPW];
+#pragma unroll
+        for (int i = 0; i < KPW; i++) {
+            const int k = wave + NW * i;
+            e_lo[i] = k < KV ? s_nbr[lane * KV + k] : -1;
+            e_hi[i] = k < KV ? s_nbr[(lane + kWave) * KV + k] : -1;
         }
-        if (tid < 2) s_cov[tid] = nc > 0 ? sc.rmask[tid] : 0ull;
+#pragma unroll
+        for (int i = 0; i < KPW; i++) {
+            const int k = wave + NW * i;
+            const int c = __popcll(__ballot(e_lo[i] >= 0)) + __popcll(__ballot(e_hi[i] >= 0));
+            if (lane == 0 && k < KV) s_cnt[k] = c;
+        }
         lds_barrier();
-    } else {
-        // the conv wave reads the groups back from the book: the stores have left this CU once every wave has
-        // waited for its own (the barrier below does), and the book's lines are in no cache of this CU yet
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __syncthreads();
+        const int mine = lane < KV ? (s_cnt[lane] + SPH_GROUP - 1) / SPH_GROUP : 0; // groups of offset `lane`
+        const int incl = wave_inclusive_sum(lane == kc ? 0 : mine);
+        const int nc = __builtin_amdgcn_readlane(mine, kc);
+        n0 = __builtin_amdgcn_readlane(incl, kWave - 1);
+        ngrp = n0 + nc;
+        fits = ngrp <= kFusedGroups;
+        if (fits) {
+            const int first = lane == kc ? n0 : incl - mine; // first group of offset `lane`
+#pragma unroll
+            for (int i = 0; i < KPW; i++) {
+                const int k = wave + NW * i;
+                if (k >= KV) break;
+                const unsigned long long b_lo = __ballot(e_lo[i] >= 0), b_hi = __ballot(e_hi[i] >= 0);
+                const int g0 = __builtin_amdgcn_readlane(first, k), ng = __builtin_amdgcn_readlane(mine, k);
+                const int below = __builtin_amdgcn_mbcnt_hi((unsigned)(b_lo >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b_lo, 0));
+                const int below_hi = __builtin_amdgcn_mbcnt_hi((unsigned)(b_hi >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b_hi, 0));
+                if (e_lo[i] >= 0) {
+                    const int d = g0 * SPH_GROUP + below;
+                    m_gat[d] = e_lo[i];
+                    m_own[d] = (unsigned char)lane;
+                }
+                if (e_hi[i] >= 0) {
+                    const int d = g0 * SPH_GROUP + __popcll(b_lo) + below_hi;
+                    m_gat[d] = e_hi[i];
+                    m_own[d] = (unsigned char)(lane + kWave);
+                }
+                if (lane < ng) m_gk[g0 + lane] = (unsigned char)k;
+                if (k == kc && lane == 0) {
+                    s_cov[0] = b_lo;
+                    s_cov[1] = b_hi;
+                }
+            }
+            if (nc == 0 && tid < 2) s_cov[tid] = 0ull;
+            lds_barrier();
+        }
+    }
+    if (fa.write_book || !fits) {
+        // the book is wanted, or the tile has more groups than region B holds: lists and group descriptors as
+        // build_book_kernel makes them, stored to the book
+        ngrp = emit_lists<NT>(s_nbr, KV, sc, kc);
+        fits = ngrp <= kFusedGroups;
+        const int gc_lo = sc.goff[kc], nc = sc.goff[kc + 1] - gc_lo;
+        n0 = ngrp - nc;
+        if (fa.write_book && b.book.tile_nbr) emit_nbr_store(s_nbr, KV, tile, b.book, tid, NT);
+        emit_store(s_nbr, r0, KV, tile, b.cap, sc, b.book, tid, NT);
+        if (fits) {
+            // one thread per slot: descriptor -> row -> table entry, as the store to the book does
+            for (int s = tid; s < ngrp * SPH_GROUP; s += NT) {
+                const int g = s / SPH_GROUP;
+                const int info = sc.ginfo[g];
+                const int k = info & 0xff, j = ((info >> 8) & 0xff) + (s & (SPH_GROUP - 1));
+                const int row = j < (info >> 16) ? sc.sel[k * R + j] : -1;
+                const int gpos = g < gc_lo ? g : (g < gc_lo + nc ? n0 + (g - gc_lo) : g - nc);
+                const int d = gpos * SPH_GROUP + (s & (SPH_GROUP - 1));
+                m_gat[d] = row >= 0 ? s_nbr[row * KV + k] : -1;
+                m_own[d] = (unsigned char)(row >= 0 ? row : 0);
+                if ((s & (SPH_GROUP - 1)) == 0) m_gk[gpos] = (unsigned char)k;
+            }
+            if (tid < 2) s_cov[tid] = nc > 0 ? sc.rmask[tid] : 0ull;
+            lds_barrier();
+        } else {
+            // the conv wave reads the groups back from the book: the stores have left this CU once every wave has
+            // waited for its own (the barrier below does), and the book's lines are in no cache of this CU yet
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __syncthreads();
+        }
     }
 
     // 2. region A becomes the accumulator tile: the helper waves store the middle offset's products into it (and
