@@ -215,17 +215,30 @@ def test_extension_functions_match_reference_signatures():
     many = np.repeat(idx[:1], 50000, axis=0)
     with pytest.raises(ValueError, match="duplicate"):
         ext.init_tensor(G.t(np.zeros((50000, 2), np.float32)), G.t(many), 2, [8, 9, 9])
+    # the same mistakes on a grid deep enough for the bitmap path
+    deep = idx.copy(); deep[:, 3] = deep[:, 3] * 30 + 7
+    ext.init_tensor(G.t(feat), G.t(deep), 2, [8, 9, 300])
+    with pytest.raises(ValueError, match="duplicate"):
+        ext.init_tensor(G.t(np.concatenate([feat, feat[:1]])), G.t(np.concatenate([deep, deep[:1]])), 2, [8, 9, 300])
+    bad = deep.copy(); bad[0, 3] = 300
+    with pytest.raises(ValueError):
+        ext.init_tensor(G.t(feat), G.t(bad), 2, [8, 9, 300])
+    with pytest.raises(ValueError, match="duplicate"):
+        ext.init_tensor(G.t(np.zeros((50000, 2), np.float32)), G.t(np.repeat(deep[:1], 50000, axis=0)), 2, [8, 9, 300])
 
 
 @pytest.mark.parametrize("B,shape,n", [(1, (64, 512, 32), 40000), (3, (7, 5, 3), 50), (2, (2048, 2048, 1024), 3000),
                                        (1, (4, 4, 4), 0), (1, (1, 1, 1), 1), (2, (8, 8, 64), 6000),
                                        (1, (16, 16, 128), 20000), (1, (16, 16, 129), 20000), (1, (3, 3, 200), 0),
-                                       (1, (1024, 1024, 16), 150000), (2, (512, 300, 130), 90000)])
+                                       (1, (1024, 1024, 16), 150000), (2, (512, 300, 130), 90000),
+                                       (1, (8, 8, 300), 15000), (2, (5, 7, 64 * 3), 6000)])
 def test_init_tensor_sizes(B, shape, n):
-    """COO -> compressed layout at sizes that need more than 32 key bits, one cell, no voxel
-    at all, long fibers, either side of the depth (128 bins) at which rows are sorted instead of
-    ranked inside their column, and column counts whose scan looks back over more than 64 workgroups
-    (sum scan: 1M columns; max scan: 307k); checked against the oracle and against the defining invariants."""
+    """COO -> compressed layout at sizes whose cells need more than 32 bits, one cell, no voxel
+    at all, long fibers, either side of the depth (128 bins) from which a row's rank comes from its column's
+    bitmap instead of a walk over the column's rows, deep grids that are nearly full (columns of hundreds of rows),
+    a deep grid whose bitmap would exceed the library's limit (2048 x 2048 x 1024: ranked by the walk), and column
+    counts whose scan looks back over more than 64 workgroups (1M and 307k columns); checked against the oracle
+    and against the defining invariants."""
     rng = np.random.default_rng(B * 1000 + n)
     cells = B * shape[0] * shape[1] * shape[2]
     lin = np.unique(rng.integers(0, cells, size=n, dtype=np.int64))[:n] if n else np.zeros(0, np.int64)
