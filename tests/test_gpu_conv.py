@@ -380,7 +380,7 @@ def _full_size_case(cfg):
 
 
 @pytest.mark.parametrize("cfg,ic,oc,dtype,backward", [
-    (2, 32, 32, torch.float16, False), (3, 32, 64, torch.float16, False), (5, 64, 64, torch.float16, True),
+    (2, 32, 32, torch.float16, False), (3, 32, 64, torch.float16, True), (5, 64, 64, torch.float16, True),
     (2, 64, 64, torch.float16, True),      # the shape the benchmark times: configuration 2's grid at 64 -> 64
     (2, 64, 64, torch.bfloat16, True), (3, 32, 64, torch.bfloat16, False)],
     ids=["cfg2-32-32-f16", "cfg3-32-64-f16", "cfg5b-64-64-f16", "headline-64-64-f16", "headline-64-64-bf16",
@@ -388,7 +388,7 @@ def _full_size_case(cfg):
 def test_configs_full_size_fp16(cfg, ic, oc, dtype, backward):
     """BASELINE configurations 2, 3, 5b and the benchmark's shape (configuration 2's grid, 64 -> 64) at full
     size: fp16 / bf16 storage with fp32 accumulate against the C oracle (fp32) on the same rounded inputs;
-    5b and the benchmark's shape also dgrad and wgrad."""
+    3 (fp16), 5b and the benchmark's shape also dgrad and wgrad."""
     d, book, (oz_idx, _, rules, rule_size, _) = _full_size_case(cfg)
     rng = np.random.default_rng(cfg)
     n, m = d["z_idx"].shape[0], oz_idx.shape[0]
@@ -406,7 +406,7 @@ def test_configs_full_size_fp16(cfg, ic, oc, dtype, backward):
     g = torch.tensor(rng.standard_normal((m, oc)), dtype=torch.float32).to(dtype)
     w_perm = w.permute(0, 2, 1).contiguous()
     d_feat, d_w = ext.rule_conv_backward(g.to(G.DEV), feat.to(G.DEV), w_perm.to(G.DEV), book, None, [1, 1])
-    tgs = [-(-d["spatial_shape"][0] // 2), -(-d["spatial_shape"][1] // 2)]
+    tgs = [-(-book.out_shape[0] // 2), -(-book.out_shape[1] // 2)]    # tiles of 2 x 2 output columns
     df_o, dw_o = O.rule_conv_backward(g.float().numpy(), feat.float().numpy(), w_perm.float().numpy(), rules,
                                       rule_size, tgs)
     assert (np.abs(d_feat.float().cpu().numpy() - df_o) <= ulp * np.abs(df_o) + 1e-3).all()
