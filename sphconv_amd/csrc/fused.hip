@@ -77,8 +77,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(NT == 256 ? 
     const int kc = KV / 2;
     int ngrp = 0, n0 = 0;
     bool fits = false;
-    if (!fa.write_book) {
-        // Nobody wants the book: the groups go from the table straight to region B.  A wave takes the offsets
+    {
+        // The groups go from the table straight to region B.  A wave takes the offsets
         // wave, wave + NW, ...: the table's column of an offset stays in two registers per lane (rows lane and
         // lane + 64), two ballots count its pairs; behind one barrier every wave knows all counts, hence where an
         // offset's groups start, and a row's rank in its offset's list (the bits below it in the ballots) is its
@@ -133,38 +133,42 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(NT == 256 ? 
             }
             if (nc == 0 && tid < 2) s_cov[tid] = 0ull;
             lds_barrier();
+            if (fa.write_book) {
+                // The book is wanted too (a shared indice_key, a backward pass): region B holds all of it.  Region B
+                // keeps the middle offset's groups last, the book keeps them in place: group p of region B is group
+                // p (offsets below the middle), p + nc (offsets above it) or p - n0 + gc_lo (the middle's own).
+                const int gc_lo = __builtin_amdgcn_readlane(incl, kc); // groups of the offsets below the middle one
+                const long gbase = (long)tile * b.cap;
+                if (b.book.tile_nbr) emit_nbr_store(s_nbr, KV, tile, b.book, tid, NT);
+                if (wave == 0) {
+                    uint16_t *koff = b.book.tile_koff + (long)tile * (KV + 1);
+                    if (lane < KV) koff[lane] = (uint16_t)(lane < kc ? incl - mine : (lane == kc ? gc_lo : incl - mine + nc));
+                    if (lane == 0) {
+                        koff[KV] = (uint16_t)ngrp;
+                        b.book.tile_ngrp[tile] = ngrp;
+                    }
+                }
+                for (int s = tid; s < ngrp * SPH_GROUP; s += NT) {
+                    const int p = s / SPH_GROUP;
+                    const int g = p < gc_lo ? p : (p < n0 ? p + nc : p - n0 + gc_lo);
+                    const int gi = m_gat[s], d = g * SPH_GROUP + (s & (SPH_GROUP - 1));
+                    b.book.grp_gather[gbase * SPH_GROUP + d] = gi;
+                    b.book.grp_owner[gbase * SPH_GROUP + d] = gi >= 0 ? r0 + (int)m_own[s] : -1;
+                    if ((s & (SPH_GROUP - 1)) == 0) b.book.grp_k[gbase + g] = m_gk[p];
+                }
+            }
         }
     }
-    if (fa.write_book || !fits) {
-        // the book is wanted, or the tile has more groups than region B holds: lists and group descriptors as
-        // build_book_kernel makes them, stored to the book
+    if (!fits) {
+        // the tile has more groups than region B holds: lists and group descriptors as build_book_kernel makes
+        // them, stored to the book
         ngrp = emit_lists<NT>(s_nbr, KV, sc, kc);
-        fits = ngrp <= kFusedGroups;
-        const int gc_lo = sc.goff[kc], nc = sc.goff[kc + 1] - gc_lo;
-        n0 = ngrp - nc;
         if (fa.write_book && b.book.tile_nbr) emit_nbr_store(s_nbr, KV, tile, b.book, tid, NT);
         emit_store(s_nbr, r0, KV, tile, b.cap, sc, b.book, tid, NT);
-        if (fits) {
-            // one thread per slot: descriptor -> row -> table entry, as the store to the book does
-            for (int s = tid; s < ngrp * SPH_GROUP; s += NT) {
-                const int g = s / SPH_GROUP;
-                const int info = sc.ginfo[g];
-                const int k = info & 0xff, j = ((info >> 8) & 0xff) + (s & (SPH_GROUP - 1));
-                const int row = j < (info >> 16) ? sc.sel[k * R + j] : -1;
-                const int gpos = g < gc_lo ? g : (g < gc_lo + nc ? n0 + (g - gc_lo) : g - nc);
-                const int d = gpos * SPH_GROUP + (s & (SPH_GROUP - 1));
-                m_gat[d] = row >= 0 ? s_nbr[row * KV + k] : -1;
-                m_own[d] = (unsigned char)(row >= 0 ? row : 0);
-                if ((s & (SPH_GROUP - 1)) == 0) m_gk[gpos] = (unsigned char)k;
-            }
-            if (tid < 2) s_cov[tid] = nc > 0 ? sc.rmask[tid] : 0ull;
-            lds_barrier();
-        } else {
-            // the conv wave reads the groups back from the book: the stores have left this CU once every wave has
-            // waited for its own (the barrier below does), and the book's lines are in no cache of this CU yet
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-            __syncthreads();
-        }
+        // the conv wave reads the groups back from the book: the stores have left this CU once every wave has
+        // waited for its own (the barrier below does), and the book's lines are in no cache of this CU yet
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
     }
 
     // 2. region A becomes the accumulator tile: the helper waves store the middle offset's products into it (and
