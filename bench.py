@@ -423,7 +423,7 @@ def record_traffic(fetch_csv, write_csv, seed, voxels):
     for n in sizes:
         blocks = ((n + 127) // 128 + 7) // 8 * 8        # tiles, rounded up to whole rounds over the 8 XCDs
         tiles = (n + 127) // 128
-        wanted = {"conv": ("conv_wave_kernel", lambda g: g == blocks * 64),
+        wanted = {"conv": ("conv_wave_run_kernel", lambda g: g == blocks * 192),   # wave 0 + two helper waves per tile
                   "rules": ("build_book_kernel<false>", lambda g: g == blocks * 256),
                   # one launch: workgroups of 256 threads up to 768 tiles, of 128 beyond
                   "rules_conv": ("rules_conv_kernel", lambda g: g == blocks * (256 if tiles <= 768 else 128))}
@@ -620,7 +620,7 @@ class Workload:
         """(the step's dominant kernel, the rule kernel, the convolution kernel): algorithmic bytes per launch over
         the kernel's average duration, against the HBM peak."""
         rules = self._roofline("build_book_kernel<false>", "rules", self.rule_bytes, kern["rulegen_ms"], seed)
-        conv = self._roofline("conv_wave_kernel<f16,2,4,false>", "conv", self.conv_bytes, kern["conv_forward_ms"], seed)
+        conv = self._roofline("conv_wave_run_kernel<f16,2,4,false>", "conv", self.conv_bytes, kern["conv_forward_ms"], seed)
         if self.one_launch:
             name = "rules_conv_kernel<f16,2,4,false,%d>" % (256 if self.ntiles <= 768 else 128)
             main = self._roofline(name, "rules_conv", self.fused_bytes, kern["rules_conv_one_launch_ms"], seed)

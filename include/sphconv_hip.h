@@ -95,6 +95,11 @@ typedef struct sph_book {
      * it can walk by rows (rows of 16-byte multiples up to 128 bytes) and refuses the others,
      * sph_conv_wgrad and sph_rules_to_padded_count refuse the book. */
     int32_t *tile_nbr;
+    /* Set by the caller, read by sph_conv_apply: not 0 = the middle offset KV/2 holds a run of full groups in most
+     * tiles, as in a submanifold layer, where it pairs every row with itself (and in that layer's transposed book).
+     * The grouped kernel then gives that run to helper waves, which load its weight fragments once.  0 (also what
+     * a zero-initialised struct says): no assumption; results are the same either way, up to the order of summation. */
+    int32_t middle_run;
 } sph_book;
 
 const char *sph_last_error(void);

@@ -36,7 +36,7 @@ class Geom(C.Structure):
 class Book(C.Structure):
     _fields_ = [("tile_ngrp", C.c_void_p), ("tile_koff", C.c_void_p), ("grp_k", C.c_void_p),
                 ("grp_gather", C.c_void_p), ("grp_owner", C.c_void_p), ("rows", C.c_int32),
-                ("KV", C.c_int32), ("tile_nbr", C.c_void_p)]
+                ("KV", C.c_int32), ("tile_nbr", C.c_void_p), ("middle_run", C.c_int32)]
 
 
 class Epilogue(C.Structure):
@@ -44,7 +44,7 @@ class Epilogue(C.Structure):
 
 
 _lib = None
-ABI_VERSION = 6       # sph_abi_version() of the library these signatures describe
+ABI_VERSION = 7       # sph_abi_version() of the library these signatures describe
 
 _I, _P, _L, _Z = C.c_int, C.c_void_p, C.c_long, C.c_size_t
 _SIGNATURES = {

@@ -135,10 +135,54 @@ __global__ __launch_bounds__(128) void conv_wave_kernel(ConvArgs a, int nwtot)
     if (r0 >= a.book.rows) return;
     const int nrows = min(R, a.book.rows - r0);
     const int col0 = wave * CT * 16;           // first column of this wave
-    const int ngrp = a.book.tile_ngrp[tile];
+    const int ngrp = min(max(a.book.tile_ngrp[tile], 0), a.cap);
     const BookMeta meta(a.book, a.cap, tile, ngrp, r0, nrows, a.feat_rows);
     conv_wave_groups<DT, NS, CT, MASKED>(a, nwtot, meta, ngrp, s_acc, col0, lane, true);
     conv_wave_store<DT, CT>(a, nwtot, s_acc, col0, r0, nrows, lane, kWave);
+}
+
+// The same with two helper waves per tile (up to 64 output columns, rows of up to 128 bytes).  A submanifold book
+// has a run of up to eight full groups at the middle offset (every row's pair with itself), which all use one set
+// of weight fragments: the helper waves load those fragments once, take the run's groups between them, multiply
+// from zero and store the products to the owners' accumulator rows behind wave 0's clear and before its first
+// sum, while wave 0's first rows and fragments are on their way.  Wave 0's chain is then the tile's other groups
+// only (26 instead of 34 at LiDAR sparsity), and the run costs 8 fragment loads instead of 64.  A tile whose middle
+// offset holds fewer than two groups (strided books) is wave 0's alone, and the helper waves leave at once.
+constexpr int kRunHelpers = 2;
+template <sph_dtype DT, int NS, int CT, bool MASKED>
+__global__ __launch_bounds__(kWave * (1 + kRunHelpers)) __attribute__((amdgpu_waves_per_eu(3))) void conv_wave_run_kernel(ConvArgs a, int nwtot)
+{
+    extern __shared__ __attribute__((aligned(16))) uint32_t s_acc[]; // [R + 1][LDW]
+    constexpr int kRun = (R / SPH_GROUP + kRunHelpers - 1) / kRunHelpers;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int tile = sph_xcd_tile(blockIdx.x, (a.book.rows + R - 1) / R);
+    const int r0 = tile * R;
+    if (r0 >= a.book.rows) return;
+    const int nrows = min(R, a.book.rows - r0);
+    const int KV = a.book.KV, kc = KV / 2;
+    const int ngrp = min(max(a.book.tile_ngrp[tile], 0), a.cap);
+    const unsigned short *ko = a.book.tile_koff + (long)tile * (KV + 1) + kc;
+    const int run_lo = min((int)ko[0], ngrp);
+    const int run_n = min(max((int)ko[1] - run_lo, 0), min(ngrp - run_lo, R / SPH_GROUP));
+    const bool shared = run_n >= 2; // workgroup-uniform
+    if (wave == 0) {
+        const BookMeta meta(a.book, a.cap, tile, shared ? ngrp - run_n : ngrp, r0, nrows, a.feat_rows, run_lo, shared ? run_n : 0);
+        conv_wave_groups<DT, NS, CT, MASKED>(a, nwtot, meta, meta.ngrp, s_acc, 0, lane, true, shared ? 2 : 0);
+    } else {
+        if (!shared) return;
+        const BookMeta meta(a.book, a.cap, tile, ngrp, r0, nrows, a.feat_rows);
+        conv_run_store<DT, NS, CT, MASKED, kRun>(a, nwtot, meta, kc, run_lo + wave - 1, kRunHelpers, run_lo + run_n, lane, s_acc,
+                                                 nullptr, -1, 0, true);
+        lds_barrier();
+    }
+    if (shared) { // the helper waves have waited for the tile: all three write it out
+        lds_barrier();
+        conv_wave_store<DT, CT>(a, nwtot, s_acc, 0, r0, nrows, tid, kWave * (1 + kRunHelpers));
+    } else {
+        conv_wave_store<DT, CT>(a, nwtot, s_acc, 0, r0, nrows, lane, kWave);
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -1143,6 +1187,17 @@ int launch_conv_wave(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
 {
     size_t lds = (size_t)(R + 1) * (nwtot * 16 + 4) * sizeof(uint32_t); // + scratch row
     const int waves = (nwtot + CT - 1) / CT;
+    if constexpr (NS <= 2 && !(DT == SPH_F32 && NS == 2 && CT == 4)) {
+        // one wave's worth of columns, rows of up to 128 bytes: helper waves for the middle offset's run (fp32 rows
+        // of 128 bytes into 64 columns do not fit the registers three waves per SIMD leave)
+        if (waves == 1 && a.book.tile_koff && a.book.middle_run) {
+            int rc = set_lds(conv_wave_run_kernel<DT, NS, CT, MASKED>, lds);
+            if (rc) return rc;
+            hipLaunchKernelGGL((conv_wave_run_kernel<DT, NS, CT, MASKED>), dim3(sph_xcd_grid(ntiles)), dim3(kWave * (1 + kRunHelpers)),
+                               lds, st, a, nwtot);
+            return sph_check_launch("sph_conv_apply");
+        }
+    }
     int rc = set_lds(conv_wave_kernel<DT, NS, CT, MASKED>, lds);
     if (rc) return rc;
     hipLaunchKernelGGL((conv_wave_kernel<DT, NS, CT, MASKED>), dim3(sph_xcd_grid(ntiles)), dim3(waves * kWave), lds, st, a, nwtot);

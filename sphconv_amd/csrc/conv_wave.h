@@ -183,30 +183,42 @@ constexpr int kRsrcFlags = 0x00020000; // raw buffer descriptor, 32-bit data for
 struct BookMeta {
     __amdgpu_buffer_rsrc_t r_gat, r_own, r_gk;
     int cap, ngrp, r0, nrows, feat_rows, KV;
-    __device__ __forceinline__ BookMeta(const sph_book &book, int cap_, int tile, int ngrp_, int r0_, int nrows_, int feat_rows_)
-        : cap(cap_), ngrp(ngrp_), r0(r0_), nrows(nrows_), feat_rows(feat_rows_), KV(book.KV)
+    int skip_lo, skip_n; // groups [skip_lo, skip_lo + skip_n) of the book are somebody else's: group g >= skip_lo is the book's g + skip_n
+    __device__ __forceinline__ BookMeta(const sph_book &book, int cap_, int tile, int ngrp_, int r0_, int nrows_, int feat_rows_,
+                                        int skip_lo_ = 0, int skip_n_ = 0)
+        : cap(cap_), ngrp(ngrp_), r0(r0_), nrows(nrows_), feat_rows(feat_rows_), KV(book.KV), skip_lo(skip_lo_), skip_n(skip_n_)
     {
         const long gb0 = (long)tile * cap;
         r_gat = __builtin_amdgcn_make_buffer_rsrc((void *)(book.grp_gather + gb0 * SPH_GROUP), 0, cap * SPH_GROUP * 4, kRsrcFlags);
         r_own = __builtin_amdgcn_make_buffer_rsrc((void *)(book.grp_owner + gb0 * SPH_GROUP), 0, cap * SPH_GROUP * 4, kRsrcFlags);
         r_gk = __builtin_amdgcn_make_buffer_rsrc((void *)(book.grp_k + gb0), 0, cap * 4, kRsrcFlags);
     }
+    __device__ __forceinline__ int book_group(int g) const { return min(g < skip_lo ? g : g + skip_n, cap - 1); }
     __device__ __forceinline__ void load(int g0, int lane, int &gi, int &ow, int &kk) const
     {
-        const int gs = min(g0, cap - kBlk); // stay inside this tile's capacity
-        gi = __builtin_amdgcn_raw_buffer_load_b32(r_gat, lane * 4, gs * (SPH_GROUP * 4), 0);
-        ow = __builtin_amdgcn_raw_buffer_load_b32(r_own, lane * 4, gs * (SPH_GROUP * 4), 0);
-        kk = __builtin_amdgcn_raw_buffer_load_b32(r_gk, (lane & (kBlk - 1)) * 4, gs * 4, 0);
+        // lane l: entry l % 16 of group g0 + l / 16, inside this tile's capacity
+        const int slot = (book_group(g0 + (lane >> 4)) * SPH_GROUP + (lane & 15)) * 4;
+        gi = __builtin_amdgcn_raw_buffer_load_b32(r_gat, slot, 0, 0);
+        ow = __builtin_amdgcn_raw_buffer_load_b32(r_own, slot, 0, 0);
+        kk = __builtin_amdgcn_raw_buffer_load_b32(r_gk, book_group(g0 + (lane & (kBlk - 1))) * 4, 0, 0);
     }
     __device__ __forceinline__ void finish(int g0, int lane, int &gi, int &ow, int &kk) const
     {
-        const bool inside = g0 <= cap - kBlk;
         const int g = g0 + (lane >> 4);
         const int vow = ow - r0;
-        const bool ok = inside && g < ngrp && (unsigned)vow < (unsigned)nrows && (unsigned)gi < (unsigned)feat_rows;
+        const bool ok = g < ngrp && (unsigned)vow < (unsigned)nrows && (unsigned)gi < (unsigned)feat_rows;
         gi = ok ? gi : -1;
         ow = ok ? vow : -1;
-        kk = (inside && g0 + (lane & (kBlk - 1)) < ngrp && (unsigned)kk < (unsigned)KV) ? kk : 0;
+        kk = (g0 + (lane & (kBlk - 1)) < ngrp && (unsigned)kk < (unsigned)KV) ? kk : 0;
+    }
+    // one slot of a run of groups (conv_run_store): gathered row or -1, owner row inside the tile
+    __device__ __forceinline__ void slot(int s, int &gi, int &ow) const
+    {
+        const int off = min(s, cap * SPH_GROUP - 1) * 4;
+        gi = __builtin_amdgcn_raw_buffer_load_b32(r_gat, off, 0, 0);
+        ow = __builtin_amdgcn_raw_buffer_load_b32(r_own, off, 0, 0) - r0;
+        const bool ok = (unsigned)ow < (unsigned)nrows && (unsigned)gi < (unsigned)feat_rows;
+        gi = ok ? gi : -1;
     }
 };
 
@@ -231,6 +243,11 @@ struct LdsMeta {
         ow = ok ? ow : -1;
         kk = (inside && g0 + (lane & (kBlk - 1)) < ngrp) ? kk : 0;
     }
+    __device__ __forceinline__ void slot(int s, int &gi, int &ow) const
+    {
+        gi = gat[s];
+        ow = own[s];
+    }
 };
 
 // Clears the wave's CT*16 columns of the accumulator tile (and of the scratch row behind it).
@@ -243,7 +260,8 @@ __device__ __forceinline__ void conv_wave_clear(uint32_t *s_acc, int LDW, int co
 
 // The tile's groups, one after the other, into the wave's columns [col0, col0 + CT*16) of s_acc ([R + 1][LDW]
 // 32-bit words, cleared by the caller, by clear() below while the first indices are on their way, or by the other
-// waves of the workgroup meanwhile: wait_clear then makes this wave meet them at a barrier before its first sum).
+// waves of the workgroup meanwhile: wait_clear then makes this wave meet them at that many barriers before its first
+// sum).
 //
 // One group: the accumulator rows of the group's owners are requested first and are the C operand of the MFMAs
 // (the matrix unit does the addition; adding the products with the vector ALU instead was measured 6 % slower:
@@ -255,7 +273,7 @@ __device__ __forceinline__ void conv_wave_clear(uint32_t *s_acc, int LDW, int co
 // issued together, so no group waits for a permute of its own.
 template <sph_dtype DT, int NS, int CT, bool MASKED, class Meta>
 __device__ __forceinline__ void conv_wave_groups(const ConvArgs &a, int nwtot, const Meta &meta, int ngrp, uint32_t *s_acc,
-                                                 int col0, int lane, bool clear, bool wait_clear = false)
+                                                 int col0, int lane, bool clear, int wait_clear = 0)
 {
     typedef typename Traits<DT>::acc4 acc4;
     const int LDW = nwtot * 16 + 4;
@@ -364,7 +382,9 @@ __device__ __forceinline__ void conv_wave_groups(const ConvArgs &a, int nwtot, c
         load_a(r3, a_3);
         __builtin_amdgcn_sched_barrier(0);
     }
-    if (wait_clear) lds_barrier(); // the other waves of the workgroup have prepared the tile meanwhile
+    // the other waves of the workgroup prepare the tile meanwhile: they start behind the first barrier (the tile is
+    // clear by then) or have started already, and are done at the last
+    for (int i = 0; i < wait_clear; i++) lds_barrier();
     for (int g0 = 0; g0 < ngrp; g0 += kBlk) {
         ow_c = ow_n; k_c = k_n;
         gi_n = gi_nn; ow_n = ow_nn; k_n = k_nn;
@@ -386,10 +406,10 @@ __device__ __forceinline__ void conv_wave_groups(const ConvArgs &a, int nwtot, c
 // Owner rows of one offset's groups are all different, so the helper waves' stores never meet (the scratch row
 // takes the padding slots of all of them, and is never read for a result).  Rows without a pair at this offset
 // (bit clear in `covered`, two 64-bit words) are zeroed by the thread that `zrow` names (-1: none).
-template <sph_dtype DT, int NS, int CT, bool MASKED, int kRunGroups>
-__device__ __forceinline__ void conv_run_store(const ConvArgs &a, int nwtot, const LdsMeta &m, int k, int g_first, int g_step,
+template <sph_dtype DT, int NS, int CT, bool MASKED, int kRunGroups, class Meta>
+__device__ __forceinline__ void conv_run_store(const ConvArgs &a, int nwtot, const Meta &m, int k, int g_first, int g_step,
                                                int g_end, int lane, uint32_t *s_acc, const unsigned long long *covered, int zrow,
-                                               int zrow_step)
+                                               int zrow_step, bool wait_clear = false)
 {
     typedef typename Traits<DT>::acc4 acc4;
     const int LDW = nwtot * 16 + 4;
@@ -397,18 +417,11 @@ __device__ __forceinline__ void conv_run_store(const ConvArgs &a, int nwtot, con
     const int wstep = nwtot * (kWave * 16);
     const __amdgpu_buffer_rsrc_t r_w = __builtin_amdgcn_make_buffer_rsrc((void *)a.wp, 0, a.book.KV * NS * wstep, kRsrcFlags);
     int4v fw[NS][CT], fa[kRunGroups][NS];
-    int ow[kRunGroups];
+    int ow[kRunGroups], gi[kRunGroups];
 #pragma unroll
     for (int j = 0; j < kRunGroups; j++) {
         const int g = g_first + j * g_step;
-        const int slot = min(g, g_end - 1) * SPH_GROUP + (lane & 15);
-        const int gi = m.gat[slot];
-        const bool ok = g < g_end && gi >= 0;
-        ow[j] = ok ? (int)m.own[slot] : R;
-        const int row_off = (int)__umul24((unsigned)(ok ? gi : 0), (unsigned)a.row_bytes) + (lane >> 4) * 16;
-#pragma unroll
-        for (int st = 0; st < NS; st++)
-            fa[j][st] = __builtin_bit_cast(int4v, __builtin_amdgcn_raw_buffer_load_b128(r_feat, row_off + st * 64, 0, 0));
+        m.slot(min(g, g_end - 1) * SPH_GROUP + (lane & 15), gi[j], ow[j]);
     }
 #pragma unroll
     for (int st = 0; st < NS; st++)
@@ -416,10 +429,21 @@ __device__ __forceinline__ void conv_run_store(const ConvArgs &a, int nwtot, con
         for (int c = 0; c < CT; c++)
             fw[st][c] = __builtin_bit_cast(int4v, __builtin_amdgcn_raw_buffer_load_b128(r_w, st * wstep + c * (kWave * 16) + lane * 16,
                                                                                           k * (NS * wstep), 0));
+#pragma unroll
+    for (int j = 0; j < kRunGroups; j++) {
+        const bool ok = g_first + j * g_step < g_end && gi[j] >= 0;
+        ow[j] = ok ? ow[j] : R;
+        const int row_off = (int)__umul24((unsigned)(ok ? gi[j] : 0), (unsigned)a.row_bytes) + (lane >> 4) * 16;
+#pragma unroll
+        for (int st = 0; st < NS; st++)
+            fa[j][st] = __builtin_bit_cast(int4v, __builtin_amdgcn_raw_buffer_load_b128(r_feat, row_off + st * 64, 0, 0));
+    }
     // rows the offset does not reach start from zero (while the loads are on their way)
-    for (int r = zrow; r >= 0 && r < R; r += zrow_step)
-        if (!((covered[r >> 6] >> (r & 63)) & 1ull))
-            for (int i = 0; i < LDW / 4; i++) ((int4v *)(s_acc + r * LDW))[i] = int4v{0, 0, 0, 0};
+    if (covered)
+        for (int r = zrow; r >= 0 && r < R; r += zrow_step)
+            if (!((covered[r >> 6] >> (r & 63)) & 1ull))
+                for (int i = 0; i < LDW / 4; i++) ((int4v *)(s_acc + r * LDW))[i] = int4v{0, 0, 0, 0};
+    if (wait_clear) lds_barrier(); // somebody else clears the tile: not before that
 #pragma unroll
     for (int j = 0; j < kRunGroups; j++) {
         acc4 prod[CT];

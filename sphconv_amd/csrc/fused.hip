@@ -178,7 +178,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(NT == 256 ? 
     if (fits) {
         if (wave == 0) {
             const LdsMeta meta{m_gat, m_own, m_gk, kFusedGroups, n0};
-            conv_wave_groups<DT, NS, CT, MASKED>(a, fa.nwtot, meta, n0, s_mem, 0, lane, false, true);
+            conv_wave_groups<DT, NS, CT, MASKED>(a, fa.nwtot, meta, n0, s_mem, 0, lane, false, 1);
         } else {
             const LdsMeta meta{m_gat, m_own, m_gk, kFusedGroups, ngrp};
             conv_run_store<DT, NS, CT, MASKED, kRun>(a, fa.nwtot, meta, kc, n0 + wave - 1, NW - 1, ngrp, lane, s_mem, s_cov,

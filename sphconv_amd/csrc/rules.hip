@@ -395,7 +395,7 @@ void sph_set_error(const char *fmt, ...)
 }
 
 SPH_EXPORT const char *sph_last_error(void) { return g_err; }
-SPH_EXPORT int sph_abi_version(void) { return 6; }
+SPH_EXPORT int sph_abi_version(void) { return 7; }
 SPH_EXPORT int sph_book_tiles(int rows) { return rows <= 0 ? 0 : sph_div_up(rows, R); }
 SPH_EXPORT int sph_book_cap(int KV) { return KV * (R / SPH_GROUP); }
 

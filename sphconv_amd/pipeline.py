@@ -53,6 +53,8 @@ class ScanPipeline:
         self._epi = L.Epilogue(None, None, 0)
         self._streams = [torch.cuda.Stream(device=dev) for _ in range(int(streams))]
         self._books = [_Buffers(self.max_voxels, self.kv, dev) for _ in self._streams]
+        for book in self._books:
+            book.struct().middle_run = 1              # submanifold: every row pairs with itself at the middle offset
         self._packed = torch.empty(nbytes, dtype=torch.uint8, device=dev)
         self._packed_ready = torch.cuda.Event()
         self.fused = bool(fused)

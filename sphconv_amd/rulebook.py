@@ -46,7 +46,7 @@ class _Buffers:
         ptrs = [base + o for o in self._off]
         if not self.groups:
             ptrs[2] = ptrs[3] = ptrs[4] = None
-        self._struct = L.Book(*ptrs[:5], self.rows, self.kv, ptrs[5] if by_row else None)
+        self._struct = L.Book(*ptrs[:5], self.rows, self.kv, ptrs[5] if by_row else None, 0)
         self._views = {}
 
     def struct(self) -> L.Book:
@@ -184,6 +184,7 @@ class RuleBook:
                 by_row = est >= BY_ROW_MIN_PAIRS * BY_ROW_FORWARD_ONLY
             groups = not (by_row and forward_only)
         buf = _Buffers(rows, self.kv, self.z_ptr.device, by_row, groups)
+        buf.struct().middle_run = int(self.subm)     # every row pairs with itself at the middle offset
         g, b = self.geom(), buf.struct()
         lib = L.lib()
         hint = _row_cols_ptr(self.row_cols if transposed else self.out_row_cols, rows)
@@ -386,6 +387,7 @@ class RuleBook:
         if not feature.is_contiguous():
             feature = feature.contiguous()
         buf = buffers if buffers is not None else _Buffers(self.out_rows, self.kv, self.z_ptr.device)
+        buf.struct().middle_run = int(self.subm)
         if out is None:
             out = torch.empty((self.out_rows, ndim), dtype=feature.dtype, device=feature.device)
         g = self.geom()
