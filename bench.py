@@ -510,6 +510,8 @@ class Workload:
         torch = self.torch
         from sphconv_amd.pipeline import ScanPipeline
         pipe = ScanPipeline(self.w, self.B, self.shape, max_voxels=self.n, streams=streams, fused=fused)
+        if fused:
+            self.step_launches = pipe.launches_for(self.n)    # what the timed step of `value` is made of
 
         def submit(k):
             feat, z_idx, z_ptr, cols = self.scans[k % len(self.scans)]
@@ -621,7 +623,7 @@ class Workload:
         the kernel's average duration, against the HBM peak."""
         rules = self._roofline("build_book_kernel<false>", "rules", self.rule_bytes, kern["rulegen_ms"], seed)
         conv = self._roofline("conv_wave_run_kernel<f16,2,4,false>", "conv", self.conv_bytes, kern["conv_forward_ms"], seed)
-        if self.one_launch:
+        if self.one_launch and getattr(self, "step_launches", 1) == 1:
             name = "rules_conv_kernel<f16,2,4,false,%d>" % (256 if self.ntiles <= 768 else 128)
             main = self._roofline(name, "rules_conv", self.fused_bytes, kern["rules_conv_one_launch_ms"], seed)
         else:
@@ -632,7 +634,8 @@ class Workload:
         """Matrix-unit figures of the convolution: useful flops (2 x pairs x iC x oC) over the kernel's duration
         against the fp16 MFMA peak, and what the kernel executes for them (whole groups of 16 pairs: the padding
         slots of a group are multiplied too)."""
-        ms = kern.get("rules_conv_one_launch_ms", kern["conv_forward_ms"]) if self.one_launch else kern["conv_forward_ms"]
+        one = self.one_launch and getattr(self, "step_launches", 1) == 1
+        ms = kern.get("rules_conv_one_launch_ms", kern["conv_forward_ms"]) if one else kern["conv_forward_ms"]
         groups = self.executed_groups
         executed = 2.0 * groups * 16 * self.ic * self.oc
         return {"useful_flops": self.flops, "executed_flops": executed, "executed_over_useful": executed / self.flops,
@@ -691,7 +694,7 @@ def main():
         return {"ms_per_step": t["ms"], "host_ms_per_step": t["host_ms"],
                 "one_stream_ms_per_step": t["one_stream_ms"], "one_stream_host_ms_per_step": t["one_stream_host_ms"],
                 "two_launch_ms_per_step": t["two_launch_ms"], "two_launch_host_ms_per_step": t["two_launch_host_ms"],
-                "launches_per_step": 1 if wl.one_launch else 2,
+                "launches_per_step": getattr(wl, "step_launches", 1 if wl.one_launch else 2),
                 "rulegen_ms_per_scan": kern["rulegen_ms"], "kernels": kern, "roofline": main_roof,
                 "roofline_rules": rules_roof, "roofline_conv": conv_roof, "mfma": wl.mfma(kern), "repeats": t["repeats"]}
 

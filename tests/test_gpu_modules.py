@@ -174,6 +174,7 @@ def test_scan_pipeline_matches_the_plain_path():
     for fused in (True, False):
         pipe = ScanPipeline(w, B, shape, max_voxels=4096, streams=3, fused=fused)
         assert pipe.streams == 3
+        assert pipe.launches_for(4096) == (1 if fused else 2) and pipe.launches_for(128 * 769) == 2
         scans = []
         for s in range(7):                                     # more scans than slots, different sizes
             idx, feat = _inputs(10 + s, B, shape, ic, p=0.1 + 0.05 * s)
