@@ -86,9 +86,15 @@ def event_ms(fn, iters, torch):
     overlaps with the previous call's execution."""
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
-    for _ in range(3):
-        fn()
-    torch.cuda.synchronize()
+    # untimed calls first, for at least 30 ms: the chip's clocks take some tens of milliseconds of one kernel's
+    # load to settle (the first 200 launches of a 20 us kernel read 5-7 % slower than those 25 ms later)
+    t0 = time.perf_counter()
+    while True:
+        for _ in range(max(3, iters)):
+            fn()
+        torch.cuda.synchronize()
+        if time.perf_counter() - t0 >= 0.03:
+            break
     start.record()
     for _ in range(iters):
         fn()

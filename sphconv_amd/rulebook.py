@@ -386,7 +386,12 @@ class RuleBook:
             return None
         if not feature.is_contiguous():
             feature = feature.contiguous()
-        buf = buffers if buffers is not None else _Buffers(self.out_rows, self.kv, self.z_ptr.device)
+        if buffers is not None:
+            buf = buffers
+        elif self.keep:
+            buf = _Buffers(self.out_rows, self.kv, self.z_ptr.device)
+        else:
+            buf = _scratch_book(self.out_rows, self.kv, self.z_ptr.device)   # nobody keeps it: the stream's own
         buf.struct().middle_run = int(self.subm)
         if out is None:
             out = torch.empty((self.out_rows, ndim), dtype=feature.dtype, device=feature.device)
@@ -518,6 +523,25 @@ def _pinned_word():
 def _release_pinned_word(word):
     if len(_PINNED_WORDS) < 64:
         _PINNED_WORDS.append(word)
+
+
+# Scratch books of one-launch calls that keep no book (the kernel still wants one for tiles with more groups than
+# its LDS holds): one per device, stream and kernel volume, grown on demand.  Calls on one stream run one after the
+# other, so they can share it; calls on different streams get different ones.
+_SCRATCH_BOOKS = {}
+
+
+def _scratch_book(rows: int, kv: int, device) -> "_Buffers":
+    key = (device.index, L.stream(), kv)
+    buf = _SCRATCH_BOOKS.get(key)
+    if buf is None or buf.capacity < rows:
+        if len(_SCRATCH_BOOKS) >= 64:
+            _SCRATCH_BOOKS.clear()
+        buf = _Buffers(max(rows, 1 << 17), kv, device)
+        buf.capacity = buf.rows
+        _SCRATCH_BOOKS[key] = buf
+    buf.struct().rows = rows
+    return buf
 
 
 def _row_cols_ptr(row_cols, rows: int):
