@@ -1223,7 +1223,7 @@ int launch_conv_wave_ct(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st
         // are faster (configuration 5a: 50.5 -> 45.5 us); with 128-byte fp16 rows they are slower (123 -> 151 us)
         // (up to 64 output columns only: more would be four waves, beyond the kernel's launch bound)
         if constexpr (DT == SPH_I8)
-            if (ntiles > 1024 && nwtot <= 4) return launch_conv_wave_m<DT, NS, 2>(a, nwtot, ntiles, st);
+            if (ntiles > 1024 && nwtot <= 4 && !a.book.middle_run) return launch_conv_wave_m<DT, NS, 2>(a, nwtot, ntiles, st);
         return launch_conv_wave_m<DT, NS, 4>(a, nwtot, ntiles, st);
     }
 }
