@@ -195,12 +195,14 @@ def encoder_stack_ms(torch, seed, iters):
     rng = np.random.default_rng(seed)
     feat = torch.tensor(rng.standard_normal((n, 16)), dtype=torch.float32, device=dev).half()
     z_idx, z_ptr = torch.tensor(d["z_idx"], device=dev), torch.tensor(d["z_ptr"], device=dev)
+    from sphconv_amd.rulebook import row_columns
+    cols = row_columns(z_ptr, n)         # part of the tensor, as init_tensor leaves it
     net = encoder_stack(16, (16, 32, 64, 64), seed=seed).to(dev).half()
     res = {"batch": B, "voxels_in": n}
 
     def one():
         with torch.no_grad():
-            return net(sphconv.SparseConvTensor(feat, shape, B, z_idx=z_idx, z_ptr=z_ptr))
+            return net(sphconv.SparseConvTensor(feat, shape, B, z_idx=z_idx, z_ptr=z_ptr, row_cols=cols))
 
     for fused in (True, False, True, False):             # each mode twice, the faster repeat counts
         net.fuse_eval = fused

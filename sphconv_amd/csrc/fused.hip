@@ -20,7 +20,7 @@
 
 namespace {
 
-constexpr int kFusedGroups = 64; // groups of a tile that region B holds (a LiDAR-like tile has 30 to 45)
+constexpr int kFusedGroups = kCompactGroups; // groups of a tile that region B holds (a LiDAR-like tile has 30 to 45)
 
 struct FusedArgs {
     BuildArgs b;
@@ -36,7 +36,7 @@ inline size_t fused_region_a(int KV, int nwtot)
     const size_t tab = (size_t)R * KV * sizeof(int32_t) + emit_scratch_bytes(KV);
     return ((acc > tab ? acc : tab) + 15) & ~(size_t)15;
 }
-inline size_t fused_region_b() { return (size_t)kFusedGroups * SPH_GROUP * 5 + kFusedGroups; }
+inline size_t fused_region_b() { return compact_bytes(); }
 
 
 // NT threads per workgroup: 256 (four waves: more hands for the rule generation, at most three workgroups per CU
@@ -64,100 +64,23 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(NT == 256 ? 
     unsigned char *m_own = (unsigned char *)(m_gat + kFusedGroups * SPH_GROUP);
     unsigned char *m_gk = m_own + kFusedGroups * SPH_GROUP;
     __shared__ unsigned long long s_cov[2];
-    __shared__ int s_cnt[32];
-
-    // region B starts as "no pair anywhere": the direct compaction below writes the slots that hold one
-    for (int i = tid; i < kFusedGroups * SPH_GROUP / 4; i += NT) ((int4v *)m_gat)[i] = int4v{-1, -1, -1, -1};
 
     // 1. the tile's pairs: the table of (row, offset) -> gathered row
     tile_table<false, false, NT>(b, tile, s_nbr, nullptr);
-    // The groups of the middle offset (in a submanifold layer: every row's pair with itself, a run of eight full
-    // groups) go to the waves that would otherwise wait, and are the first the tile is given: stored, not added.
-    // The compact arrays keep them behind the other groups.
+    // 2. the groups, from the table straight to region B (compact_groups).  Those of the middle offset (in a
+    // submanifold layer: every row's pair with itself, a run of eight full groups) go to the waves that would
+    // otherwise wait, and are the first the tile is given: stored, not added.  Region B keeps them behind the
+    // other groups.
     const int kc = KV / 2;
-    int ngrp = 0, n0 = 0;
-    bool fits = false;
-    {
-        // The groups go from the table straight to region B.  A wave takes the offsets
-        // wave, wave + NW, ...: the table's column of an offset stays in two registers per lane (rows lane and
-        // lane + 64), two ballots count its pairs; behind one barrier every wave knows all counts, hence where an
-        // offset's groups start, and a row's rank in its offset's list (the bits below it in the ballots) is its
-        // slot.  Rows ascending inside an offset, offsets ascending, the middle offset last: the order of the lists
-        // that emit_lists makes, without the lists.
-        constexpr int KPW = (32 + NW - 1) / NW; // KV <= 32
-        int e_lo[KPW], e_hi[KPW];
-#pragma unroll
-        for (int i = 0; i < KPW; i++) {
-            const int k = wave + NW * i;
-            e_lo[i] = k < KV ? s_nbr[lane * KV + k] : -1;
-            e_hi[i] = k < KV ? s_nbr[(lane + kWave) * KV + k] : -1;
-        }
-#pragma unroll
-        for (int i = 0; i < KPW; i++) {
-            const int k = wave + NW * i;
-            const int c = __popcll(__ballot(e_lo[i] >= 0)) + __popcll(__ballot(e_hi[i] >= 0));
-            if (lane == 0 && k < KV) s_cnt[k] = c;
-        }
-        lds_barrier();
-        const int mine = lane < KV ? (s_cnt[lane] + SPH_GROUP - 1) / SPH_GROUP : 0; // groups of offset `lane`
-        const int incl = wave_inclusive_sum(lane == kc ? 0 : mine);
-        const int nc = __builtin_amdgcn_readlane(mine, kc);
-        n0 = __builtin_amdgcn_readlane(incl, kWave - 1);
-        ngrp = n0 + nc;
-        fits = ngrp <= kFusedGroups;
-        if (fits) {
-            const int first = lane == kc ? n0 : incl - mine; // first group of offset `lane`
-#pragma unroll
-            for (int i = 0; i < KPW; i++) {
-                const int k = wave + NW * i;
-                if (k >= KV) break;
-                const unsigned long long b_lo = __ballot(e_lo[i] >= 0), b_hi = __ballot(e_hi[i] >= 0);
-                const int g0 = __builtin_amdgcn_readlane(first, k), ng = __builtin_amdgcn_readlane(mine, k);
-                const int below = __builtin_amdgcn_mbcnt_hi((unsigned)(b_lo >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b_lo, 0));
-                const int below_hi = __builtin_amdgcn_mbcnt_hi((unsigned)(b_hi >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b_hi, 0));
-                if (e_lo[i] >= 0) {
-                    const int d = g0 * SPH_GROUP + below;
-                    m_gat[d] = e_lo[i];
-                    m_own[d] = (unsigned char)lane;
-                }
-                if (e_hi[i] >= 0) {
-                    const int d = g0 * SPH_GROUP + __popcll(b_lo) + below_hi;
-                    m_gat[d] = e_hi[i];
-                    m_own[d] = (unsigned char)(lane + kWave);
-                }
-                if (lane < ng) m_gk[g0 + lane] = (unsigned char)k;
-                if (k == kc && lane == 0) {
-                    s_cov[0] = b_lo;
-                    s_cov[1] = b_hi;
-                }
-            }
-            if (nc == 0 && tid < 2) s_cov[tid] = 0ull;
-            lds_barrier();
-            if (fa.write_book) {
-                // The book is wanted too (a shared indice_key, a backward pass): region B holds all of it.  Region B
-                // keeps the middle offset's groups last, the book keeps them in place: group p of region B is group
-                // p (offsets below the middle), p + nc (offsets above it) or p - n0 + gc_lo (the middle's own).
-                const int gc_lo = __builtin_amdgcn_readlane(incl, kc); // groups of the offsets below the middle one
-                const long gbase = (long)tile * b.cap;
-                if (b.book.tile_nbr) emit_nbr_store(s_nbr, KV, tile, b.book, tid, NT);
-                if (wave == 0) {
-                    uint16_t *koff = b.book.tile_koff + (long)tile * (KV + 1);
-                    if (lane < KV) koff[lane] = (uint16_t)(lane < kc ? incl - mine : (lane == kc ? gc_lo : incl - mine + nc));
-                    if (lane == 0) {
-                        koff[KV] = (uint16_t)ngrp;
-                        b.book.tile_ngrp[tile] = ngrp;
-                    }
-                }
-                for (int s = tid; s < ngrp * SPH_GROUP; s += NT) {
-                    const int p = s / SPH_GROUP;
-                    const int g = p < gc_lo ? p : (p < n0 ? p + nc : p - n0 + gc_lo);
-                    const int gi = m_gat[s], d = g * SPH_GROUP + (s & (SPH_GROUP - 1));
-                    b.book.grp_gather[gbase * SPH_GROUP + d] = gi;
-                    b.book.grp_owner[gbase * SPH_GROUP + d] = gi >= 0 ? r0 + (int)m_own[s] : -1;
-                    if ((s & (SPH_GROUP - 1)) == 0) b.book.grp_k[gbase + g] = m_gk[p];
-                }
-            }
-        }
+    const CompactGroups cg{m_gat, m_own, m_gk};
+    const CompactInfo ci = compact_groups<NT>(s_nbr, KV, kc, cg, s_cov);
+    int ngrp = ci.ngrp;
+    const int n0 = ci.n0;
+    const bool fits = ci.fits;
+    if (fits && fa.write_book) {
+        // the book is wanted too (a shared indice_key, a backward pass): region B holds all of it
+        if (b.book.tile_nbr) emit_nbr_store(s_nbr, KV, tile, b.book, tid, NT);
+        compact_store<NT>(cg, ci, kc, r0, KV, tile, b.cap, b.book);
     }
     if (!fits) {
         // the tile has more groups than region B holds: lists and group descriptors as build_book_kernel makes
@@ -171,9 +94,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(NT == 256 ? 
         __syncthreads();
     }
 
-    // 2. region A becomes the accumulator tile: the helper waves store the middle offset's products into it (and
+    // 3. region A becomes the accumulator tile: the helper waves store the middle offset's products into it (and
     //    zero the rows that offset does not reach) while wave 0 requests its first rows and fragments;
-    // 3. wave 0 adds the other groups one after the other.
+    // 4. wave 0 adds the other groups one after the other.
     const int LDW = fa.nwtot * 16 + 4;
     if (fits) {
         if (wave == 0) {
@@ -195,7 +118,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(NT == 256 ? 
     }
     lds_barrier();
 
-    // 4. the tile goes to global memory once, by all threads, with the epilogue fused
+    // 5. the tile goes to global memory once, by all threads, with the epilogue fused
     conv_wave_store<DT, CT>(a, fa.nwtot, s_mem, 0, r0, nrows, tid, NT);
 }
 

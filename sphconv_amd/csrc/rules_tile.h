@@ -129,7 +129,10 @@ __host__ __device__ inline size_t emit_scratch_bytes(int KV)
     size_t b = (size_t)KV * sizeof(int) + (size_t)(KV + 1) * sizeof(int) + (size_t)KV * (R / SPH_GROUP) * sizeof(int);
     b = (b + 7) & ~(size_t)7;
     b += 2 * sizeof(unsigned long long) + (size_t)KV * R;
-    return (b + 7) & ~(size_t)7;
+    b = (b + 7) & ~(size_t)7;
+    // the compact copy of a tile's groups (compact_groups below) takes the same place
+    const size_t compact = (size_t)64 * SPH_GROUP * 5 + 64;
+    return b > compact ? b : compact;
 }
 // `base` must be 8-byte aligned.
 __device__ __forceinline__ EmitScratch emit_scratch_at(void *base, int KV)
@@ -269,6 +272,125 @@ __device__ __forceinline__ void emit_nbr_store(const int32_t *nbr, int KV, int t
     }
 }
 
+// ---------------------------------------------------------------------------
+// The tile's groups from the table straight to a compact copy in LDS, without lists (kernel volumes of up to 32,
+// tiles of up to kCompactGroups groups).  A wave takes the offsets wave, wave + NW, ...: an offset's column of the
+// table is two registers per lane (rows lane and lane + 64), two ballots count its pairs; behind one barrier every
+// wave reads all counts and scans them in its own registers, so it knows where every offset's groups start, and a
+// row's rank in its offset's list (the ballot bits below it) is its slot.  Rows ascending inside an offset, offsets
+// ascending: the order emit_lists + emit_store produce, at two barriers instead of five and without the chain
+// descriptor -> row -> table entry per slot.  k_last >= 0 puts that offset's groups behind all others (the
+// one-launch kernel gives them to other waves); rows with a pair at k_last are reported in s_cov (two words).
+// ---------------------------------------------------------------------------
+constexpr int kCompactGroups = 64;
+struct CompactGroups {
+    int32_t *gat;            // [kCompactGroups * SPH_GROUP] gathered row or -1
+    unsigned char *own, *gk; // [kCompactGroups * SPH_GROUP] owner row inside the tile; [kCompactGroups] offset of the group
+};
+__host__ __device__ inline size_t compact_bytes() { return (size_t)kCompactGroups * SPH_GROUP * 5 + kCompactGroups; }
+__device__ __forceinline__ CompactGroups compact_at(void *base) // 16-byte aligned
+{
+    CompactGroups cg;
+    cg.gat = (int32_t *)base;
+    cg.own = (unsigned char *)(cg.gat + kCompactGroups * SPH_GROUP);
+    cg.gk = cg.own + kCompactGroups * SPH_GROUP;
+    return cg;
+}
+struct CompactInfo {
+    int ngrp, n0, nc; // groups of the tile; of all offsets but k_last; of k_last (0 without one)
+    int gc_lo;        // groups of the offsets below k_last
+    int first;        // per lane: first group, in the book's order, of offset `lane`
+    bool fits;        // ngrp <= kCompactGroups: the compact copy was written
+};
+template <int NT>
+__device__ __forceinline__ CompactInfo compact_groups(const int32_t *nbr, int KV, int k_last, const CompactGroups &cg,
+                                                      unsigned long long *s_cov)
+{
+    static_assert(R == 2 * kWave, "two ballots cover a tile's rows");
+    constexpr int NW = NT / kWave;
+    constexpr int KPW = (32 + NW - 1) / NW; // KV <= 32
+    __shared__ int s_cnt[32];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    for (int i = tid; i < kCompactGroups * SPH_GROUP / 4; i += NT) ((int4 *)cg.gat)[i] = make_int4(-1, -1, -1, -1);
+    int e_lo[KPW], e_hi[KPW];
+#pragma unroll
+    for (int i = 0; i < KPW; i++) {
+        const int k = wave + NW * i;
+        e_lo[i] = k < KV ? nbr[lane * KV + k] : -1;
+        e_hi[i] = k < KV ? nbr[(lane + kWave) * KV + k] : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < KPW; i++) {
+        const int k = wave + NW * i;
+        const int c = __popcll(__ballot(e_lo[i] >= 0)) + __popcll(__ballot(e_hi[i] >= 0));
+        if (lane == 0 && k < KV) s_cnt[k] = c;
+    }
+    lds_barrier();
+    CompactInfo ci;
+    const int mine = lane < KV ? (s_cnt[lane] + SPH_GROUP - 1) / SPH_GROUP : 0; // groups of offset `lane`
+    const int incl = wave_inclusive_sum(lane == k_last ? 0 : mine);
+    ci.nc = k_last >= 0 ? __builtin_amdgcn_readlane(mine, max(k_last, 0)) : 0;
+    ci.n0 = __builtin_amdgcn_readlane(incl, kWave - 1);
+    ci.ngrp = ci.n0 + ci.nc;
+    ci.gc_lo = k_last >= 0 ? __builtin_amdgcn_readlane(incl, max(k_last, 0)) : ci.n0;
+    ci.first = lane < k_last || k_last < 0 ? incl - mine : (lane == k_last ? ci.gc_lo : incl - mine + ci.nc);
+    ci.fits = ci.ngrp <= kCompactGroups;
+    if (!ci.fits) return ci;
+    const int place = lane == k_last ? ci.n0 : incl - mine; // first group of offset `lane` in the compact copy
+#pragma unroll
+    for (int i = 0; i < KPW; i++) {
+        const int k = wave + NW * i;
+        if (k >= KV) break;
+        const unsigned long long b_lo = __ballot(e_lo[i] >= 0), b_hi = __ballot(e_hi[i] >= 0);
+        const int g0 = __builtin_amdgcn_readlane(place, k), ng = __builtin_amdgcn_readlane(mine, k);
+        if (e_lo[i] >= 0) {
+            const int d = g0 * SPH_GROUP + __builtin_amdgcn_mbcnt_hi((unsigned)(b_lo >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b_lo, 0));
+            cg.gat[d] = e_lo[i];
+            cg.own[d] = (unsigned char)lane;
+        }
+        if (e_hi[i] >= 0) {
+            const int d = g0 * SPH_GROUP + __popcll(b_lo) +
+                          __builtin_amdgcn_mbcnt_hi((unsigned)(b_hi >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b_hi, 0));
+            cg.gat[d] = e_hi[i];
+            cg.own[d] = (unsigned char)(lane + kWave);
+        }
+        if (lane < ng) cg.gk[g0 + lane] = (unsigned char)k;
+        if (s_cov && k == k_last && lane == 0) {
+            s_cov[0] = b_lo;
+            s_cov[1] = b_hi;
+        }
+    }
+    if (s_cov && ci.nc == 0 && tid < 2) s_cov[tid] = 0ull;
+    lds_barrier();
+    return ci;
+}
+
+// The book's part of a tile from its compact copy (compact_groups with ci.fits), by all NT threads: group p of the
+// copy is the book's group p (offsets below k_last), p + nc (offsets above it) or p - n0 + gc_lo (k_last's own).
+template <int NT>
+__device__ __forceinline__ void compact_store(const CompactGroups &cg, const CompactInfo &ci, int k_last, int r0, int KV, int tile,
+                                              int cap, const sph_book &book)
+{
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const long gbase = (long)tile * cap;
+    if (tid < kWave) {
+        uint16_t *koff = book.tile_koff + (long)tile * (KV + 1);
+        if (lane < KV) koff[lane] = (uint16_t)ci.first;
+        if (lane == 0) {
+            koff[KV] = (uint16_t)ci.ngrp;
+            book.tile_ngrp[tile] = ci.ngrp;
+        }
+    }
+    for (int s = tid; s < ci.ngrp * SPH_GROUP; s += NT) {
+        const int p = s / SPH_GROUP;
+        const int g = p < ci.gc_lo ? p : (p < ci.n0 ? p + ci.nc : p - ci.n0 + ci.gc_lo);
+        const int gi = cg.gat[s], d = g * SPH_GROUP + (s & (SPH_GROUP - 1));
+        book.grp_gather[gbase * SPH_GROUP + d] = gi;
+        book.grp_owner[gbase * SPH_GROUP + d] = gi >= 0 ? r0 + (int)cg.own[s] : -1;
+        if ((s & (SPH_GROUP - 1)) == 0) book.grp_k[gbase + g] = cg.gk[p];
+    }
+}
+
 // Everything the book keeps of one tile, from the table in LDS.
 template <int NT>
 __device__ __forceinline__ void emit_groups(const int32_t *nbr, int nrows, int r0, int KV, int tile, int cap,
@@ -276,6 +398,17 @@ __device__ __forceinline__ void emit_groups(const int32_t *nbr, int nrows, int r
 {
     if (book.tile_nbr) emit_nbr_store(nbr, KV, tile, book, threadIdx.x, NT);
     if (!book.grp_gather) return; // the caller keeps the pairs by row only: no groups, and no group counts either
+    if (KV <= 32) {
+        // the compact copy takes the place of the list scratch (and of the masks of the mask join behind it, which
+        // the table no longer needs)
+        const CompactGroups cg = compact_at(sc.cnt);
+        const CompactInfo ci = compact_groups<NT>(nbr, KV, -1, cg, nullptr);
+        if (ci.fits) { // workgroup-uniform
+            compact_store<NT>(cg, ci, -1, r0, KV, tile, cap, book);
+            return;
+        }
+        lds_barrier(); // the lists below overwrite what the other waves may still be counting from
+    }
     emit_lists<NT>(nbr, KV, sc);
     emit_store(nbr, r0, KV, tile, cap, sc, book, threadIdx.x, NT);
 }
