@@ -902,13 +902,8 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
         g0 = min((int)ko[0], a.cap);
         n = min(max((int)ko[1] - g0, 0), min(a.cap - g0, R / SPH_GROUP));
     }
-    int incl = n;
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-        int v = __shfl_up(incl, d, kWave);
-        if (lane >= d) incl += v;
-    }
-    const int total = __shfl(incl, kWave - 1, kWave);
+    const int incl = wave_inclusive_sum(n); // lane shifts of the vector ALU, no LDS round trip per step
+    const int total = __builtin_amdgcn_readlane(incl, kWave - 1);
     if (slice_step == 1 && tid < a.nslice - 1 && blockIdx.y == 0) a.flags[slot + 1 + tid] = 0; // slots nobody fills
     if (h * kWsSlice >= total) {
         if (tid == 0 && blockIdx.y == 0) a.flags[slot] = 0;
@@ -931,16 +926,19 @@ __global__ __launch_bounds__(256, 2) void wgrad_wave_kernel(WgradArgs a)
     // Per-lane constants of the row copies: which pair and 16-byte chunk each of the lane's
     // loads moves, its offset in the source row and in the staging area (-1: none).
     int pairA[MI], srcA[MI], dstA[MI], pairG[NI], srcG[NI], dstG[NI];
+    // (rows of 32, 64 or 128 bytes are 2, 4 or 8 chunks: a shift instead of the forty instructions of a division)
+    const bool p2A = (cprA & (cprA - 1)) == 0, p2G = (cprG & (cprG - 1)) == 0;
+    const int shA = __ffs(cprA) - 1, shG = __ffs(cprG) - 1;
 #pragma unroll
     for (int it = 0; it < MI; it++) {
         const int i = it * kWave + lane;
-        const int pa = i / cprA, ca = i - pa * cprA;
+        const int pa = p2A ? i >> shA : i / cprA, ca = i - pa * cprA;
         pairA[it] = min(pa, PB - 1); srcA[it] = ci0 * E + ca * 16; dstA[it] = pa < PB ? pa * rsA + ca * 16 : -1;
     }
 #pragma unroll
     for (int it = 0; it < NI; it++) {
         const int i = it * kWave + lane;
-        const int pg = i / cprG, cg = i - pg * cprG;
+        const int pg = p2G ? i >> shG : i / cprG, cg = i - pg * cprG;
         pairG[it] = min(pg, PB - 1); srcG[it] = co0 * E + cg * 16; dstG[it] = pg < PB ? pg * rsG + cg * 16 : -1;
     }
     const unsigned strideA = a.iC * E, strideG = a.oC * E;   // arrays are below 4 GiB (checked by the launcher)
