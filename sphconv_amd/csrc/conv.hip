@@ -1188,7 +1188,9 @@ int launch_conv_wave(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st)
     if constexpr (NS <= 2 && !(DT == SPH_F32 && NS == 2 && CT == 4)) {
         // one wave's worth of columns, rows of up to 128 bytes: helper waves for the middle offset's run (fp32 rows
         // of 128 bytes into 64 columns do not fit the registers three waves per SIMD leave)
-        if (waves == 1 && a.book.tile_koff && a.book.middle_run) {
+        // (narrow layers on large grids keep the one-wave kernel: a group is one fragment load and one MFMA there,
+        // and the helper waves' barriers cost a full chip more than the run saves: 16 -> 16 on 4912 tiles 22.6 / 25.8 us)
+        if (waves == 1 && a.book.tile_koff && a.book.middle_run && (NS * CT >= 4 || ntiles <= 1024)) {
             int rc = set_lds(conv_wave_run_kernel<DT, NS, CT, MASKED>, lds);
             if (rc) return rc;
             hipLaunchKernelGGL((conv_wave_run_kernel<DT, NS, CT, MASKED>), dim3(sph_xcd_grid(ntiles)), dim3(kWave * (1 + kRunHelpers)),
