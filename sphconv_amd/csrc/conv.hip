@@ -1220,8 +1220,9 @@ int launch_conv_wave_ct(const ConvArgs &a, int nwtot, int ntiles, hipStream_t st
     case 2: return launch_conv_wave_m<DT, NS, 2>(a, nwtot, ntiles, st);
     default:
         // int8 rows are 64 bytes: on a full chip two waves per tile (32 columns each, the rows gathered twice)
-        // are faster (configuration 5a: 50.5 -> 45.5 us); with 128-byte fp16 rows they are slower (123 -> 151 us)
-        // (up to 64 output columns only: more would be four waves, beyond the kernel's launch bound)
+        // are faster than one (configuration 5a: 50.5 -> 45.5 us); with 128-byte fp16 rows they are slower (123 -> 151 us)
+        // (up to 64 output columns only: more would be four waves, beyond the kernel's launch bound).  A book with a
+        // run at its middle offset takes one wave of 64 columns and two helper waves instead (5a: 36.7 -> 35.1 us).
         if constexpr (DT == SPH_I8)
             if (ntiles > 1024 && nwtot <= 4 && !a.book.middle_run) return launch_conv_wave_m<DT, NS, 2>(a, nwtot, ntiles, st);
         return launch_conv_wave_m<DT, NS, 4>(a, nwtot, ntiles, st);

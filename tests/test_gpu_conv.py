@@ -111,6 +111,55 @@ def _f64_pair_sum(case, feat64, w64, transposed=False):
     return out, absacc
 
 
+@pytest.mark.parametrize("subm,p", [(True, 0.25), (True, 0.012), (True, 0.9), (False, 0.25)])
+@pytest.mark.parametrize("dtype,ic,oc", [(torch.float32, 16, 16), (torch.float16, 64, 64), (torch.bfloat16, 32, 48),
+                                         (torch.float16, 8, 64), (torch.int8, 64, 64)])
+def test_middle_run_is_a_hint_not_a_contract(subm, p, dtype, ic, oc):
+    """sph_conv_apply with and without sph_book.middle_run (helper waves for the middle offset's groups) against the
+    oracle: submanifold books with full runs, with tiles whose middle offset holds one group or none (the helper
+    waves leave), nearly full grids (tiles of more than 64 groups), and a strided book, which has no run whatever the
+    caller claims.  Integers equal, floating point to the path's tolerance; each setting twice, bit for bit."""
+    import ctypes as C
+    from sphconv_amd import _lib as L
+    case = _random_case(int(p * 1000) + ic + 7 * oc, subm, p=p, shape=(9, 36, 20))
+    book = case["book"]
+    n, m = book.in_rows, book.out_rows
+    rng = np.random.default_rng(5)
+    if dtype == torch.int8:
+        feat = torch.tensor(rng.integers(-128, 128, (n, ic)), dtype=torch.int8)
+        w = torch.tensor(rng.integers(-128, 128, (27, ic, oc)), dtype=torch.int8)
+        scale = torch.tensor((rng.random(oc) + 0.5) / 3000.0, dtype=torch.float32)
+        want = O.rule_conv_i8(feat.numpy(), w.numpy(), scale.numpy(), case["oracle"][2], case["oracle"][3], m)
+    else:
+        feat = torch.tensor(rng.standard_normal((n, ic)), dtype=torch.float32).to(dtype)
+        w = torch.tensor(_weights(rng, 27, ic, oc)).to(dtype)
+        scale = None
+        want = _oracle_fwd(case, feat.float().numpy(), w.float().numpy())
+    feat, w = feat.to(G.DEV), w.to(G.DEV)
+    packed = ext._packed_weight(w, False)
+    sc_keep = scale.to(G.DEV) if scale is not None else None
+    epi = L.Epilogue(L.ptr(sc_keep), None, 0)
+    bk = book.fwd.struct()
+    outs = []
+    for flag in (0, 1, 0, 1):
+        bk.middle_run = flag
+        out = torch.full((m, oc), 3, device=G.DEV).to(dtype)
+        L.check(L.lib().sph_conv_apply(L.dtype_code(dtype), L.ptr(feat), n, ic, L.ptr(packed), oc, C.byref(bk), C.byref(epi),
+                                       L.ptr(out), L.stream()))
+        torch.cuda.synchronize()
+        outs.append(out)
+    bk.middle_run = int(subm)
+    assert torch.equal(outs[0], outs[2]) and torch.equal(outs[1], outs[3])
+    G.assert_same_conv(outs[0], outs[1])
+    for out in outs[:2]:
+        if dtype == torch.int8:
+            assert np.array_equal(out.cpu().numpy(), want)
+        elif dtype == torch.float32:
+            np.testing.assert_allclose(out.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
+        else:
+            np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=1e-2, atol=1e-3 * max(1.0, float(np.abs(want).max())))
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("ic,oc", [(4, 4), (16, 16), (32, 32), (32, 64), (64, 64), (24, 40), (128, 128)])
 @pytest.mark.parametrize("subm", [True, False])
