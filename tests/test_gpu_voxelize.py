@@ -83,6 +83,45 @@ def test_many_points_scan_over_many_workgroups():
     assert want["voxel_num"] > 30000
 
 
+@pytest.mark.parametrize("max_points,max_voxels", [(5, 4000), (40, 4000), (3, 300), (1, 1)])
+def test_crowded_cells_long_segments_and_the_stop(max_points, max_voxels):
+    """Synthetic cells: a third of 20 000 points share one cell and a tenth another (segments of thousands of
+    points, which a wave walks together), the rest spread over 3000 cells with hash collisions among them, one
+    point in 50 outside the grid; with 300 voxels (and with one) the reference's loop stops in the middle of the list.
+    Bit-exact against the sequential loop on the same cells."""
+    rng = np.random.default_rng(max_points * 1000 + max_voxels)
+    n, grid = 20000, [64, 64, 8]
+    ncell = grid[0] * grid[1] * grid[2]
+    pool = rng.choice(ncell, 3000, replace=False)
+    cells = pool[rng.integers(0, 3000, n)]
+    u = rng.random(n)
+    cells = np.where(u < 0.33, pool[0], np.where(u < 0.43, pool[1], cells))
+    cells = np.where(rng.random(n) < 0.02, -1, cells).astype(np.int64)
+    pts = rng.normal(0, 10, (n, 4)).astype(np.float32)
+    ok = cells >= 0
+    c = np.where(ok, cells, 0)
+    coor = np.stack([c // (grid[0] * grid[1]), c // grid[0] % grid[1], c % grid[0]], 1)
+    want = O.voxelize_cells(pts, pts, coor, ok, max_points, max_voxels, 0)
+    res = points_to_voxel_v2(pts, None, RANGE, SRANGE, None, max_points, max_voxels, resolution_HWD=grid,
+                             coord_system="spherical", append_mode=0, cells=torch.tensor(cells))
+    _compare(res, want)
+    if max_voxels == 4000:
+        assert want["voxel_num"] == np.unique(cells[ok]).size > 2500 and want["num_points_per_voxel"].max() == max_points
+
+
+def test_every_point_in_one_cell():
+    """70 000 points in a single cell: one segment, and the hash table's one slot takes every atomic."""
+    n = 70000
+    pts = np.random.default_rng(9).normal(0, 1, (n, 5)).astype(np.float32)
+    cells = np.full(n, 37, np.int64)
+    coor = np.tile(np.array([[0, 37 // 16, 37 % 16]]), (n, 1))
+    want = O.voxelize_cells(pts, pts, coor, np.ones(n, bool), 7, 10, 0)
+    res = points_to_voxel_v2(pts, None, RANGE, SRANGE, None, 7, 10, resolution_HWD=[16, 16, 4],
+                             coord_system="spherical", append_mode=0, cells=torch.tensor(cells))
+    _compare(res, want)
+    assert want["voxel_num"] == 1 and want["num_points_per_voxel"][0] == 7
+
+
 def test_small_and_degenerate_inputs():
     pts = np.array([[20, 1, 0.2, 0.5], [20, 1, 0.2, 0.6], [0, 0, 3, 0.1], [0, 0, 0, 0.2], [1e3, 5, 1, 0.3],
                     [30, -2, -1, 0.4], [20, 1, 0.2, 0.7]], np.float32)
