@@ -583,10 +583,11 @@ def test_forward_only_book_builds_its_groups_on_demand(pair_form):
 
 @pytest.mark.parametrize("p,shape,ic,oc,dtype", [(0.5, [24, 96, 16], 32, 32, torch.float16), (1.0, [18, 64, 16], 16, 64, torch.float16),
                                                  (0.08, [64, 256, 24], 32, 16, torch.float16), (0.5, [24, 96, 16], 16, 16, torch.float32),
-                                                 (0.6, [24, 80, 16], 64, 32, torch.int8)])
+                                                 (0.6, [24, 80, 16], 64, 32, torch.int8),
+                                                 (0.5, [24, 96, 16], 16, 32, torch.float16), (0.5, [24, 96, 16], 8, 24, torch.bfloat16)])
 def test_by_row_equals_groups_on_large_grids(monkeypatch, p, shape, ic, oc, dtype):
-    """More than 1024 tiles (one wave per tile in the by-row kernel), dense to sparse, rows of 32 and 64
-    bytes: same pairs as the grouped kernel, forward and dgrad (int8 equal; floating point to the path's tolerance:
+    """More than 1024 tiles (one wave per tile in the by-row kernel), dense to sparse, rows of 16, 32 and 64
+    bytes (up to 32 bytes in 16-bit types: two kernel offsets per MFMA, forward or dgrad): same pairs as the grouped kernel, forward and dgrad (int8 equal; floating point to the path's tolerance:
     the two kernels add a row's products in different orders)."""
     from sphconv_amd import rulebook
     from sphconv_amd.rulebook import RuleBook
