@@ -14,7 +14,9 @@ of its work into per-stream buffers, the kernels of one scan run beside those of
 `one_stream_ms_per_step` is the same step with one scan at a time through the extension's
 Python API.  The steps walk through --scans resident copies of the scan (more memory than the
 last-level cache holds); the timed loop of --steps steps is repeated --repeats times and the
-median counts, after the per-kernel section has settled the device.  `ms_per_step` is device
+median counts; the untimed steps in front of a timed loop are --warmup steps and then more of
+the same until --settle-ms have passed (the chip's clocks take tens of milliseconds of load to
+settle, a timed loop of 20 steps lasts 0.4 ms).  `ms_per_step` is device
 time (HIP events on the streams: last end - first start), `host_ms_per_step` the host's clock
 around the same region between device synchronisations.
 
@@ -44,6 +46,8 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--settle-ms", type=float, default=30.0,
+                    help="untimed warm-up steps go on until this much time has passed (clocks settle); 0: only --warmup steps")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--streams", type=int, default=3, help="HIP streams the timed scans are dealt to")
     ap.add_argument("--scans", type=int, default=24,
@@ -490,12 +494,25 @@ class Workload:
         book.keep = False
         return book, ext.rule_conv(feat, self.w, book, None, self.n, cache_packed=True)
 
-    def time_one_stream(self, steps, warmup, repeats):
+    def warm(self, submit, warmup, settle_ms):
+        """The untimed steps in front of a timed region: `warmup` of them, and more of the same until
+        `settle_ms` have passed (the chip's clocks take some tens of milliseconds of load to settle; a timed
+        region of 20 steps lasts 0.4 ms)."""
+        torch = self.torch
+        t0 = time.perf_counter()
+        done = 0
+        while True:
+            for i in range(max(warmup, 20)):
+                submit(done + i)
+            done += max(warmup, 20)
+            torch.cuda.synchronize()
+            if (time.perf_counter() - t0) * 1e3 >= settle_ms:
+                return
+
+    def time_one_stream(self, steps, warmup, repeats, settle_ms=0.0):
         torch = self.torch
         with torch.no_grad():
-            for i in range(warmup):
-                self.step(i)
-            torch.cuda.synchronize()
+            self.warm(self.step, warmup, settle_ms)
             times, dev_times = [], []
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             for r in range(repeats):
@@ -509,7 +526,7 @@ class Workload:
                 dev_times.append(e0.elapsed_time(e1) / steps)
         return sorted(dev_times)[len(dev_times) // 2], sorted(times)[len(times) // 2], dev_times
 
-    def time_pipelined(self, steps, warmup, repeats, streams, fused=True):
+    def time_pipelined(self, steps, warmup, repeats, streams, fused=True, settle_ms=0.0):
         """The same step per scan, scans dealt to a few HIP streams so that the kernels of one scan run beside
         those of another (a 100k-voxel scan does not fill the chip); buffers are allocated once per stream slot,
         every step redoes all the work.  Device time of a repeat: from the first start to the last end over the
@@ -525,10 +542,8 @@ class Workload:
             feat, z_idx, z_ptr, cols = self.scans[k % len(self.scans)]
             return pipe.submit(feat, z_idx, z_ptr, wait_inputs=False, row_cols=cols)   # inputs are resident and complete
 
-        for i in range(warmup):
-            submit(i)
+        self.warm(submit, warmup, settle_ms)
         pipe.synchronize()
-        torch.cuda.synchronize()
         ns = pipe.streams
         ref = torch.cuda.Event(enable_timing=True)
         heads = [torch.cuda.Event(enable_timing=True) for _ in range(ns)]
@@ -686,13 +701,12 @@ def main():
 
     def measure(d):
         wl = Workload(torch, d, ic, oc, w, args.scans, args.seed)
-        # the per-kernel section goes first: its hundreds of launches settle clocks and caches, so that a short
-        # timed run (--steps 20) reads the same as a long one
+        # the per-kernel section goes first (each kernel alone, behind 30 ms of its own launches)
         iters = max(100, min(args.steps, 200))
         kern = wl.time_kernels(iters, backward=args.backward, rng=rng)
-        one_dev, one_host, one_all = wl.time_one_stream(args.steps, max(args.warmup, 20), args.repeats)
-        ms, host_ms, ms_all = wl.time_pipelined(args.steps, max(args.warmup, 20), args.repeats, args.streams)
-        two = wl.time_pipelined(args.steps, max(args.warmup, 20), args.repeats, args.streams, fused=False)
+        one_dev, one_host, one_all = wl.time_one_stream(args.steps, args.warmup, args.repeats, args.settle_ms)
+        ms, host_ms, ms_all = wl.time_pipelined(args.steps, args.warmup, args.repeats, args.streams, settle_ms=args.settle_ms)
+        two = wl.time_pipelined(args.steps, args.warmup, args.repeats, args.streams, fused=False, settle_ms=args.settle_ms)
         return wl, kern, {"ms": ms, "host_ms": host_ms, "one_stream_ms": one_dev, "one_stream_host_ms": one_host,
                           "two_launch_ms": two[0], "two_launch_host_ms": two[1],
                           "repeats": {"one_stream_ms": one_all, "pipelined_ms": ms_all}}
@@ -712,7 +726,8 @@ def main():
     result = {
         "metric": "active voxels/sec, 3x3x3 subm conv 64->64 fp16 (rulegen + forward); rulegen ms/scan",
         "value": n / (rep["ms_per_step"] * 1e-3), "unit": "voxels/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": rep["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "warmup": args.warmup, "settle_ms": args.settle_ms, "ms_per_step": rep["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "config-2 generator (G2, seed %d): grid 64x2048x64, batch 1, %d active voxels, "
                                "%d pairs; subm 3x3x3 64->64, fp16 storage / fp32 accumulate; rules + forward in %d "
