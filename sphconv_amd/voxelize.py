@@ -78,7 +78,7 @@ def points_to_voxel_v2(points, voxel_size, coors_range, sphere_coors_range, coor
     voxel_num = torch.empty(1, dtype=torch.int32, device=dev)
     nbytes = lib.sph_points_to_voxel_workspace(n, grid[0], grid[1], grid[2])
     if nbytes == 0:
-        raise L.SphconvError("bad resolution %s" % (grid,))
+        raise L.SphconvError("bad resolution %s, or more than 2^29 points (%d)" % (grid, n))
     work = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     cell_out = torch.empty(n, dtype=torch.int64, device=dev) if return_cells else None
     if cells is not None:
